@@ -22,6 +22,12 @@ Families (``MODEL_REGISTRY`` keys, reference ``custom_modeling/__init__.py:4-7``
                     fp32 residual streams, optional causal input convolution, mixers ``parallel`` (sink attention
                     beside a gated delta rule) and ``lightning`` (decay linear attention), gated tanh-GELU
                     feed-forward, learned positions, untied head.
+* ``lamisun``     - per-layer description: sequential blocks whose norm sits on each sublayer's OUTPUT
+                    (x <- x + norm(sublayer(x + conv(x)))), a causal input convolution before both sublayers, the
+                    layers' results averaged over depth with learned weights, a hashed bigram row added to the
+                    embedding; mixers ``latent_attention`` (with a rotated key part shared by the heads and an output
+                    gate) and ``attention`` (two softmax maps subtracted, chunked mask, query / key norm);
+                    plain feed-forward with the xIELU activation, untied head.
 """
 from __future__ import annotations
 
@@ -46,6 +52,12 @@ class MixerSpec:
     scale: float
     window: int = 0
     kv_from: Optional[int] = None
+    # ``rot_dim`` > 0: every query head carries ``rot_dim`` more numbers after its ``dim`` and the down-projection
+    # ``rot_dim`` more rows after the latent - one key part shared by all heads - both turned by ``rot`` (pairs of
+    # neighbours) and multiplied into the score beside the latent part; the rotated key part is cached with the latent
+    rot_dim: int = 0
+    rot: Optional["RotarySpec"] = None
+    gate: bool = False  # the concatenated heads are multiplied by sigmoid(W_g h) before the output projection
 
 
 @dataclass
@@ -73,6 +85,7 @@ class RotarySpec:
     dims: int
     base: float
     scaling: Optional[tuple] = None
+    pairs: str = "half"  # "half": i with i + dims / 2; "neighbours": 2i with 2i + 1
 
 
 @dataclass
@@ -91,6 +104,34 @@ class SinkAttnSpec:
     talk: bool = False
     bias: bool = False
     kind: str = "sink_attention"
+
+
+@dataclass
+class DiffAttnSpec:
+    """Differential softmax attention over a paged key/value cache: every query head and every key head holds two
+    maps of ``dim`` numbers that attend separately over the same values (``vdim`` per key/value head); per head
+    o = a1 - lambda a2, divided by its root mean square and multiplied by 1 - ``diff``. lambda is one number of the
+    layer: exp(lq1 . lk1) - exp(lq2 . lk2) + ``diff``. ``qk_norm``: queries and keys are RMS-normed per head and map
+    with a learned weight; ``chunk`` > 0: a position sees the earlier positions of its own block of ``chunk``
+    positions only (0: all earlier positions)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    diff: float
+    chunk: int = 0
+    qk_norm: bool = True
+    kind: str = "attention"
+
+
+@dataclass
+class BigramSpec:
+    """A second embedding table of ``buckets`` + 1 rows: row (previous * mul_prev + current * mul_cur) mod buckets is
+    added to a token's embedding, the last row for a sequence's first token."""
+    buckets: int
+    mul_prev: int
+    mul_cur: int
 
 
 @dataclass
@@ -127,10 +168,12 @@ class ParallelMixerSpec:
 
 @dataclass
 class DenseMLPSpec:
-    """Gated feed-forward down(act(gate h) * (up h))."""
+    """Feed-forward down(act(gate h) * (up h)), or, ``gated`` false, down(act(up h)). ``act``: ``gelu_tanh``,
+    ``silu`` or ``xielu`` (two learned numbers per layer)."""
     ff: int
     act: str = "gelu_tanh"
     kind: str = "dense"
+    gated: bool = True
 
 
 @dataclass
@@ -178,6 +221,11 @@ class ModelConfig:
     streams: int = 0  # > 0: that many residual streams with learned read / write / mix weights per sublayer
     residual_mult: float = 1.0  # c above
     canon_taps: int = 0  # > 0: the mixer's input h becomes h + causal_conv(h) over that many taps
+    # blocks whose norm sits on the sublayer's output (x <- x + norm(sublayer(x))); the sublayers read x itself
+    post_norm: bool = False
+    canon_ffn: bool = False  # the feed-forward's input goes through an input convolution of its own as well
+    depth_average: bool = False  # what leaves layer i is a learned weighted sum of the results of layers <= i
+    bigram: Optional[BigramSpec] = None
 
     # ---------------------------------------------------------------- derived
     @property
@@ -198,10 +246,11 @@ class ModelConfig:
 
     def num_params(self) -> int:
         h, f, v = self.hidden_size, self.intermediate_size, self.vocab_size
-        if self.layer_specs and self.model_type == "babotar":
-            from .weights import babotar_shapes
+        if self.layer_specs and self.model_type in ("babotar", "lamisun"):
+            from .weights import babotar_shapes, lamisun_shapes
 
-            return sum(math.prod(shp) for shp in babotar_shapes(self).values())
+            shapes = babotar_shapes(self) if self.model_type == "babotar" else lamisun_shapes(self)
+            return sum(math.prod(shp) for shp in shapes.values())
         if self.layer_specs:
             n = v * h + h
             for s in self.layer_specs:
@@ -230,6 +279,8 @@ class ModelConfig:
             return _timisun(cls, d)
         if mt is None and d.get("architecture") == "Babotar":
             return _babotar(cls, d)
+        if mt is None and d.get("architecture") == "Lamisun":
+            return _lamisun(cls, d)
         common = dict(
             bos_token_id=d.get("bos_token_id"),
             eos_token_id=_first(d.get("eos_token_id")),
@@ -396,6 +447,57 @@ def _babotar(cls, d: Dict[str, Any]) -> "ModelConfig":
     )
 
 
+def _lamisun(cls, d: Dict[str, Any]) -> "ModelConfig":
+    """``{"architecture": "Lamisun", "vocab", "width", "norm": {"eps"}, "canon": {"taps"}, "embedding": {"scale",
+    "bigram": {"buckets", "mul_prev", "mul_cur"}}, "layers": [{"type": "latent_attention" | "attention", "mixer":
+    {...}, "mlp": {"kind": "dense", "ff"} | null}]}``. A latent mixer gives heads, dim, rot_dim, vdim, kv_rank, scale,
+    rot: {base, dims}; an attention mixer heads, kv_heads, dim, vdim, scale, diff, mask: {size}."""
+    specs: List[LayerSpec] = []
+    for i, L in enumerate(d["layers"]):
+        m, typ = L["mixer"], L.get("type")
+        if typ == "latent_attention":
+            rd = int(m.get("rot_dim") or 0)
+            rot = None
+            if rd:
+                rot = RotarySpec(int(m["rot"]["dims"]), float(m["rot"]["base"]), None, "neighbours")
+                if rot.dims != rd or rd % 2:
+                    raise ValueError(f"Lamisun layer {i}: {rot.dims} rotary dimensions on a rotated part of {rd}")
+            mixer = MixerSpec("latent_attention", int(m["heads"]), int(m["dim"]), int(m["vdim"]), int(m["kv_rank"]),
+                              float(m["scale"]), 0, None, rd, rot, True)
+        elif typ == "attention":
+            mixer = DiffAttnSpec(int(m["heads"]), int(m.get("kv_heads") or m["heads"]), int(m["dim"]), int(m["vdim"]),
+                                 float(m["scale"]), float(m["diff"]), int((m.get("mask") or {}).get("size") or 0))
+            if mixer.heads % mixer.kv_heads:
+                raise ValueError(f"Lamisun layer {i}: {mixer.heads} heads on {mixer.kv_heads} key heads")
+        else:
+            raise ValueError(f"Lamisun layer {i}: unsupported mixer type {typ!r}")
+        f, mlp = L.get("mlp"), None
+        if f is not None:
+            if f.get("kind", "dense") != "dense":
+                raise ValueError(f"Lamisun layer {i}: unsupported feed-forward kind {f.get('kind')!r}")
+            mlp = DenseMLPSpec(int(f["ff"]), "xielu", gated=False)
+        specs.append(LayerSpec(mixer, mlp))
+    if not specs:
+        raise ValueError("Lamisun: no layers")
+    emb = d.get("embedding") or {}
+    bg = emb.get("bigram")
+    bigram = None if not bg else BigramSpec(int(bg["buckets"]), int(bg["mul_prev"]), int(bg["mul_cur"]))
+    if bigram is not None and bigram.buckets < 1:
+        raise ValueError("Lamisun: the bigram table needs at least one bucket")
+    return cls(
+        model_type="lamisun", vocab_size=int(d["vocab"]), hidden_size=int(d["width"]), num_layers=len(specs),
+        num_heads=max(s.mixer.heads for s in specs), num_kv_heads=1, head_dim=1,
+        intermediate_size=max([s.mlp.ff for s in specs if s.mlp] or [0]),
+        max_position_embeddings=1 << 20,  # the design has no positional limit of its own
+        norm="rmsnorm", norm_eps=float(d["norm"]["eps"]), activation="xielu", position="none", rotary_dim=0,
+        parallel_block=False, tie_word_embeddings=False, layer_specs=specs, residual_fp32=True,
+        embedding_scale=float(emb.get("scale", 1.0)), canon_taps=int((d.get("canon") or {}).get("taps") or 0),
+        post_norm=True, canon_ffn=True, depth_average=True, bigram=bigram,
+        bos_token_id=d.get("bos_token_id"), eos_token_id=_first(d.get("eos_token_id")),
+        pad_token_id=d.get("pad_token_id"),
+    )
+
+
 def _first(x):
     if isinstance(x, (list, tuple)):
         return x[0] if x else None
@@ -483,6 +585,24 @@ _PRESETS: Dict[str, Dict[str, Any]] = {
                                   mlp=dict(kind="dense", ff=64)),
                              dict(type="lightning", mixer=dict(heads=3, dim=8, vdim=16, decay=[0.5, 0.9, 0.99]),
                                   mlp=None),
+                         ]),
+    # post-norm per-layer design: latent attention with a rotated key part and a gate, differential chunked attention
+    # with grouped heads, a layer without a feed-forward, input convolutions, depth averaging, bigram embedding
+    "tiny-lamisun": dict(architecture="Lamisun", vocab=211, width=48, norm=dict(eps=1e-5), canon=dict(taps=4),
+                         embedding=dict(scale=2.0, bigram=dict(buckets=97, mul_prev=31, mul_cur=7)),
+                         layers=[
+                             dict(type="attention",
+                                  mixer=dict(heads=4, kv_heads=2, dim=8, vdim=12, scale=0.35, diff=0.2,
+                                             mask=dict(size=12)),
+                                  mlp=dict(kind="dense", ff=80)),
+                             dict(type="latent_attention",
+                                  mixer=dict(heads=3, dim=16, rot_dim=8, vdim=12, kv_rank=24, scale=0.2,
+                                             rot=dict(base=500.0, dims=8)),
+                                  mlp=None),
+                             dict(type="latent_attention",
+                                  mixer=dict(heads=2, dim=8, rot_dim=4, vdim=16, kv_rank=20, scale=0.3,
+                                             rot=dict(base=10000.0, dims=4)),
+                                  mlp=dict(kind="dense", ff=64)),
                          ]),
     # TP up to 8 (16 q / kv heads: 2 per rank at TP=8, as Llama-2-7B's 32 give 4)
     "tiny-llama16h": dict(model_type="llama", hidden_size=256, num_hidden_layers=2, num_attention_heads=16,

@@ -1,7 +1,7 @@
 """Decoder whose layers are described one by one (``ModelConfig.layer_specs``) over an fp32 residual stream.
 
-The uniform families run through :class:`~llmss_amd.models.decoder.DecoderLM`; a per-layer design (Timisun, Babotar)
-runs through :class:`LayeredLM`, which offers the engine the same surface (``hidden_states`` / ``logits`` over a
+The uniform families run through :class:`~llmss_amd.models.decoder.DecoderLM`; a per-layer design (Timisun, Babotar,
+Lamisun) runs through :class:`LayeredLM`, which offers the engine the same surface (``hidden_states`` / ``logits`` over a
 :class:`StepInput`, ``allocate_kv_cache``, ``kv_bytes_per_block``, ``plan``) and so shares its scheduler, paged
 cache pool, decode graphs and sampler. A layer is either a parallel block (``cfg.parallel_block``)
 
@@ -11,7 +11,13 @@ or a sequential one over S residual streams x_1 .. x_S (S = 1: the ordinary pre-
 
     u = sum_s in[s] x_s ;  y = sublayer(norm(u)) ;  x_t <- sum_s mix[s, t] x_s + c * out[t] * y
 
-where the mixer may read h + causal_conv(h) instead of h. The mixer and the feed-forward are looked up by kind
+where the mixer may read h + causal_conv(h) instead of h; or (``cfg.post_norm``) a sequential block whose norm sits
+on each sublayer's output,
+
+    x <- x + norm1(mixer(x + conv1(x))) ;  x <- x + norm2(ffn(x + conv2(x)))
+
+optionally followed by a depth average: what goes on to the next layer is sum_j dwa[j] X_j over the results X_j of
+this and all earlier layers (X_0 the embedding). The mixer and the feed-forward are looked up by kind
 (``MIXERS`` / ``FFNS``), so another design can combine the same mechanisms with other constants or add its own
 beside them. Besides pages of the shared pool a mixer may own per-sequence state (a matrix state per head, the last
 inputs of a convolution): ``LayerCache.state`` tensors indexed by the scheduler's state slot of each sequence
@@ -26,7 +32,16 @@ Mixer ``latent_attention`` (ops: linear_f, latent_norm_cache, head_absorb, laten
 caches one RMS-normed latent row c per token in its paged cache ([blocks, block_size, kv_rank], the step's slots)
 and attends with the key projection absorbed into the query: qa_h = W_uk_h^T q_h, p = softmax(scale qa_h . c_j)
 over the causal (optionally windowed) keys, out = W_o concat_h(W_uv_h sum_j p_j c_j). A layer with ``kv_from``
-projects no latent of its own and reads the named layer's cache with its own W_uk / W_uv.
+projects no latent of its own and reads the named layer's cache with its own W_uk / W_uv. With ``rot_dim`` > 0 every
+query head and the cached row carry a rotated part after the latent one (the key's is shared by all heads): the score
+is the dot product over the whole row [c | k_rot], the weighted sum reads c alone. ``gate``: the heads' outputs are
+multiplied by sigmoid(W_g h) before the output projection.
+
+Mixer ``attention`` (ops: linear_f, qk_norm_cache, sink_attn without a sink, diff_combine): differential attention -
+two softmax maps per head over the same values, o = a1 - lambda a2, RMS-normed per head - with RMS-normed queries
+and keys and a chunked causal mask. The two maps of a key head are cached as two key heads; the two maps of the query
+heads of a group are laid out so that the grouped-query kernel's head mapping serves them (``vshare`` = 2: both key
+heads read one value head).
 
 Feed-forward ``moe`` (ops: moe_router -> fp32 router logits and routing, moe_experts, glu_clamp): sigmoid scores, the
 choice made on score + correction, weights = chosen scores normalised; experts and the shared expert use the clamped
@@ -53,17 +68,19 @@ class LatentAttention:
     @staticmethod
     def cache_row(spec) -> Optional[int]:
         """Numbers cached per token by a layer of this kind (None: it reads another layer's cache)."""
-        return spec.kv_rank if spec.kv_from is None else None
+        return spec.kv_rank + spec.rot_dim if spec.kv_from is None else None
 
     @staticmethod
     def forward(model: "LayeredLM", i: int, W, spec, h, inp: StepInput, cu, caches):
         dt = model.dtype
-        H, dim, R = spec.heads, spec.dim, spec.kv_rank
-        qc = ops.linear_f(h, W.qc, dt)  # [T, H * dim (+ R)]: queries, then this layer's raw latent
+        H, dim, R, rot = spec.heads, spec.dim, spec.kv_rank, spec.rot_dim
+        qc = ops.linear_f(h, W.qc, dt)  # [T, H * (dim + rot) (+ R + rot) (+ H * vdim)]: queries, raw latent, gate
         cache = caches[i if spec.kv_from is None else spec.kv_from][0]
+        qa = ops.head_absorb(qc, W.uk_t, ops.latent_qa_dtype(cache), extra=rot)
         if W.own_kv:
-            ops.latent_norm_cache(qc, H * dim, R, W.kv_norm, model.cfg.norm_eps, cache, inp.slots)
-        qa = ops.head_absorb(qc, W.uk_t, ops.latent_qa_dtype(cache))
+            cs = model.angles(inp, W.freqs) if rot else None
+            ops.latent_norm_cache(qc, H * (dim + rot), R, W.kv_norm, model.cfg.norm_eps, cache, inp.slots, rot, cs,
+                                  qa if rot else None, 0, dim)
         nd = inp.num_decode if inp.kind == "extend" else 0
         if nd and nd < qa.shape[0]:
             # mixed step: the single-token rows take the decode form of the kernel (their keys split over
@@ -78,7 +95,40 @@ class LatentAttention:
             o = ops.latent_attn(qa, cache, inp.block_tables, cu, inp.ctx_lens, spec.window, spec.scale,
                                 max_qlen=1 if single else max(1, inp.max_seqlen),
                                 max_ctx=inp.max_ctx if single else 0)
-        return ops.linear_f(ops.head_expand(o, W.uv, dt), W.o, dt)
+        y = ops.head_expand(o, W.uv, dt)
+        if W.gate_col is not None:
+            y = ops.gate_mul(y, qc, W.gate_col)
+        return ops.linear_f(y, W.o, dt)
+
+
+class DiffAttention:
+    """Mixer ``attention``: differential softmax attention over paged key / value rows."""
+
+    @staticmethod
+    def cache_row(spec) -> Optional[int]:
+        return spec.kv_heads * (2 * spec.dim + spec.vdim)
+
+    @staticmethod
+    def allocate(model: "LayeredLM", spec, num_blocks: int, block_size: int, num_slots: int):
+        dt, dev = model.dtype, model.device
+        return (torch.zeros(num_blocks, block_size, spec.kv_heads * 2 * spec.dim, dtype=dt, device=dev),
+                torch.zeros(num_blocks, block_size, spec.kv_heads * spec.vdim, dtype=dt, device=dev), {})
+
+    @staticmethod
+    def forward(model: "LayeredLM", i: int, W, spec, h, inp: StepInput, cu, caches):
+        dt, eps, c = model.dtype, model.cfg.norm_eps, W.cols
+        kc, vc = caches[i][0], caches[i][1]
+        H, G = spec.heads, spec.kv_heads
+        proj = ops.linear_f(h, W.proj, dt)
+        q = ops.qk_norm_cache(proj, c["q"], c["k"], c["v"], W.q_norm, W.k_norm, eps, kc, vc, inp.slots, H, G, 2,
+                              spec.dim, spec.vdim)
+        single = inp.kind == "decode"
+        # the two maps as 2 H query heads on 2 G key heads; both key heads of a pair read one value head
+        O = ops.sink_attn(q, kc, vc, inp.block_tables, cu, inp.ctx_lens, 2 * H, 2 * G, spec.dim, spec.vdim, spec.scale,
+                          0.0, False, max_qlen=1 if single else max(1, inp.max_seqlen),
+                          num_decode=0 if single else inp.num_decode, sink=False, chunk=spec.chunk, vshare=2)
+        y = ops.diff_combine(O, W.lam, eps, 1.0 - spec.diff, H, G, spec.vdim, dt)
+        return ops.linear_f(y, W.o, dt)
 
 
 class MoEFeedForward:
@@ -180,15 +230,18 @@ class DecayMixer:
 
 
 class DenseFeedForward:
-    """Feed-forward ``dense``: down(act(gate h) * (up h)), gate and up as one GEMM."""
+    """Feed-forward ``dense``: down(act(gate h) * (up h)), gate and up as one GEMM; ungated: down(act(up h))."""
 
     @staticmethod
     def forward(model: "LayeredLM", W, spec, h):
         dt = model.dtype
+        if not spec.gated:
+            return ops.linear_f(ops.act_fn(ops.linear_f(h, W.gu, dt), spec.act, W.act_params), W.down, dt)
         return ops.linear_f(ops.glu_act(ops.linear_f(h, W.gu, dt), spec.ff, spec.act), W.down, dt)
 
 
-MIXERS = {"latent_attention": LatentAttention, "parallel": ParallelMixer, "lightning": DecayMixer}
+MIXERS = {"latent_attention": LatentAttention, "parallel": ParallelMixer, "lightning": DecayMixer,
+          "attention": DiffAttention}
 FFNS = {"moe": MoEFeedForward, "dense": DenseFeedForward}
 
 
@@ -218,6 +271,7 @@ class LayeredLM:
         self.bucket_bytes = 0
         self.gqa_mfma: set = set()
         self._cu_decode = {}
+        self._angles = {}
         self.tap = None  # tap(i, x): called with the fp32 residual after layer i (debugging, tests)
 
     @property
@@ -266,23 +320,29 @@ class LayeredLM:
     def needs_state(self) -> bool:
         """Some mixer keeps per-sequence state besides its pages: steps must carry the sequences' state slots."""
         return any(hasattr(MIXERS[s.mixer.kind], "state_bytes") for s in self.cfg.layer_specs) or \
-            bool(self.cfg.canon_taps > 1)
+            bool(self.cfg.canon_taps > 1) or self.cfg.bigram is not None
+
+    def _canon_sublayers(self) -> int:
+        return 2 if self.cfg.canon_ffn else 1
 
     def state_bytes_per_slot(self) -> int:
         n = sum(MIXERS[s.mixer.kind].state_bytes(s.mixer) for s in self.cfg.layer_specs
                 if hasattr(MIXERS[s.mixer.kind], "state_bytes"))
-        return n + 4 * max(self.cfg.canon_taps - 1, 0) * self.cfg.hidden_size * len(self.cfg.layer_specs)
+        n += 8 if self.cfg.bigram is not None else 0
+        return n + 4 * max(self.cfg.canon_taps - 1, 0) * self.cfg.hidden_size * len(self.cfg.layer_specs) * \
+            self._canon_sublayers()
 
     def allocate_kv_cache(self, num_blocks: int, block_size: int, num_slots: int = 0):
         """One entry per layer. Latent attention: (rows, None), a layer that reads another layer's rows holding that
         layer's pair. Mixers with an ``allocate`` of their own: (key pages, value pages, {name: per-slot state});
         ``num_slots`` state slots, one per running sequence. The input convolution's tails of all layers live in
-        ``self.canon_tail`` [layers, slots, taps - 1, W]."""
+        ``self.canon_tail`` [layers (x 2 when the feed-forward has a convolution too: mixer, feed-forward), slots,
+        taps - 1, W], the token before each sequence's next one (bigram embedding) in ``self.prev_token`` [slots]."""
         caches: list = []
         for s, r in zip(self.cfg.layer_specs, self._cache_rows()):
             mx = MIXERS[s.mixer.kind]
             if hasattr(mx, "allocate"):
-                if num_slots <= 0:
+                if num_slots <= 0 and hasattr(mx, "state_bytes"):
                     raise ValueError(f"{self.cfg.model_type}: the cache needs state slots (num_slots)")
                 caches.append(mx.allocate(self, s.mixer, num_blocks, block_size, num_slots))
             elif r:
@@ -290,8 +350,11 @@ class LayeredLM:
             else:
                 caches.append(caches[s.mixer.kv_from])
         if self.cfg.canon_taps > 1:
-            self.canon_tail = torch.zeros(len(caches), max(num_slots, 1), self.cfg.canon_taps - 1,
-                                          self.cfg.hidden_size, dtype=torch.float32, device=self.device)
+            self.canon_tail = torch.zeros(len(caches) * self._canon_sublayers(), max(num_slots, 1),
+                                          self.cfg.canon_taps - 1, self.cfg.hidden_size, dtype=torch.float32,
+                                          device=self.device)
+        if self.cfg.bigram is not None:
+            self.prev_token = torch.zeros(max(num_slots, 1), dtype=torch.int64, device=self.device)
         return caches
 
     # ---------------------------------------------------------------------------- forward
@@ -315,6 +378,8 @@ class LayeredLM:
         if inp.block_tables is None or inp.ctx_lens is None or not any(t is not None for t in kv_caches[0]):
             raise ValueError(f"{self.cfg.model_type} attends through its paged cache: the step needs block tables, "
                              f"context lengths and a cache (a cache-less recompute step is not supported)")
+        if self.cfg.post_norm:
+            return self._postnorm_blocks(inp, kv_caches)
         if not self.cfg.parallel_block:
             return self._sequential_blocks(inp, kv_caches)
         cfg, w = self.cfg, self.w
@@ -360,6 +425,62 @@ class LayeredLM:
         if self.tap is not None:
             self.tap(len(w.layers) - 1, x.sum(0))
         return h
+
+    def angles(self, inp: StepInput, freqs: torch.Tensor) -> torch.Tensor:
+        """(cos, sin) [T, len(freqs), 2] of the step's positions, formed once per step and distinct rotation."""
+        key = freqs.data_ptr()
+        got = self._angles.get(key)
+        if got is None:
+            for f, cs in self._angles.values():  # another layer's table with the same steps
+                if f.shape == freqs.shape and torch.equal(f, freqs):
+                    got = (freqs, cs)
+                    break
+            if got is None:
+                got = (freqs, ops.rope_angles(inp.positions, freqs))
+            self._angles[key] = got
+        return got[1]
+
+    def _postnorm_blocks(self, inp: StepInput, kv_caches) -> torch.Tensor:
+        """Blocks normed on the sublayers' outputs, with input convolutions and the depth average. ``hist`` [L + 2,
+        T, W] fp32 holds the layers' results: layer i works in place on hist[i + 1], which the step before filled
+        with the layer's input - the embedding for layer 0, the depth average leaving layer i - 1 afterwards (without
+        depth averaging the one row block is carried along)."""
+        cfg, w, dt = self.cfg, self.w, self.dtype
+        if self.needs_state and inp.state_slots is None:
+            raise ValueError(f"{cfg.model_type} keeps per-sequence state: the step needs the sequences' state slots")
+        eps = cfg.norm_eps
+        cu = self._cu(inp)
+        T, L = inp.input_ids.shape[0], len(w.layers)
+        self._angles = {}
+        dwa = cfg.depth_average
+        hist = torch.empty(L + 2 if dwa else 2, T, cfg.hidden_size, dtype=torch.float32, device=self.device)
+        if cfg.bigram is not None:
+            ops.embed_bigram(inp.input_ids, inp.positions, w.wte, cfg.embedding_scale, w.extra["bigram"],
+                             cfg.bigram.mul_prev, cfg.bigram.mul_cur, self.prev_token, cu, inp.ctx_lens,
+                             inp.state_slots, hist)
+        else:
+            hist[0].copy_(ops.embed_scaled(inp.input_ids, w.wte, cfg.embedding_scale))
+            hist[1].copy_(hist[0])
+        nsub = self._canon_sublayers()
+        x = hist[1]
+        for i, (Lw, spec) in enumerate(zip(w.layers, cfg.layer_specs)):
+            n = i + 1 if dwa else 1
+
+            def read(canon, k):  # what a sublayer reads: x + conv(x), or x, in the storage type
+                if canon is None:
+                    return x.to(dt)
+                tail = self.canon_tail[nsub * i + k] if cfg.canon_taps > 1 else None
+                return ops.causal_conv(x, canon, tail, cu, inp.ctx_lens, inp.state_slots, True, False, dt)
+            y = MIXERS[spec.mixer.kind].forward(self, i, Lw.mix, spec.mixer, read(Lw.canon1, 0), inp, cu, kv_caches)
+            last = spec.mlp is None
+            x = ops.resid_norm_add(hist, n, y, Lw.norm1, eps, Lw.dwa if last and dwa else None)
+            if not last:
+                y = FFNS[spec.mlp.kind].forward(self, Lw.mlp, spec.mlp, read(Lw.canon2, 1))
+                x = ops.resid_norm_add(hist, n, y, Lw.norm2, eps, Lw.dwa if dwa else None)
+            if self.tap is not None:
+                self.tap(i, x)
+        self._angles = {}
+        return ops.resid_add_norm(x, None, None, w.lnf_w, 0.0, eps, dt)
 
     @property
     def vocab_lo(self) -> int:

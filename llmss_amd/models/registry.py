@@ -21,7 +21,7 @@ from ..parallel.dist import TPGroup
 from .config import ModelConfig
 from .decoder import StepInput
 from .layered import create_model
-from .weights import load_babotar_weights, load_hf_weights, load_timisun_weights
+from .weights import load_babotar_weights, load_hf_weights, load_lamisun_weights, load_timisun_weights
 
 
 @dataclass
@@ -54,8 +54,9 @@ class CausalLM:
     def __init__(self, config, weights, max_blocks: int = 4096, block_size: int = 16, max_seqs: int = 16):
         cfg = config if isinstance(config, ModelConfig) else ModelConfig.from_hf_dict(config.to_dict())
         tp = getattr(weights, "tp", None) or TPGroup()
-        if cfg.layer_specs:  # per-layer designs (Timisun, Babotar)
-            load = load_babotar_weights if cfg.model_type == "babotar" else load_timisun_weights
+        if cfg.layer_specs:  # per-layer designs (Timisun, Babotar, Lamisun)
+            load = {"babotar": load_babotar_weights, "lamisun": load_lamisun_weights}.get(cfg.model_type,
+                                                                                          load_timisun_weights)
             w = load(cfg, weights.reader, device=weights.device, dtype=weights.dtype)
         else:
             w = load_hf_weights(cfg, weights.reader, tp.size, tp.rank, device=weights.device, dtype=weights.dtype)
@@ -276,5 +277,12 @@ class BabotarForCausalLM(_FamilyLM):
     model_type = "babotar"
 
 
+class LamisunForCausalLM(_FamilyLM):
+    """Per-layer design: blocks normed on the sublayers' outputs, latent attention with a rotated key part,
+    differential chunked attention, depth-averaged layer results, bigram embedding (models/layered.py)."""
+    model_type = "lamisun"
+
+
 MODEL_REGISTRY = {c.model_type: c for c in (GPT2LMHeadModel, GPTJForCausalLM, GPTBigCodeForCausalLM,
-                                            LlamaForCausalLM, TimisunForCausalLM, BabotarForCausalLM)}
+                                            LlamaForCausalLM, TimisunForCausalLM, BabotarForCausalLM,
+                                            LamisunForCausalLM)}

@@ -162,6 +162,9 @@ def _tensors(mw: ModelWeights):
                 yield lin.b
     yield mw.lnf_w
     yield mw.head.w
+    for t in mw.extra.values():
+        if isinstance(t, torch.Tensor):
+            yield t
 
 
 # ------------------------------------------------------------------------------ finalisation
@@ -546,9 +549,14 @@ class LatentAttnWeights:
     uk_t: torch.Tensor
     uv: torch.Tensor
     o: torch.Tensor
+    # with a rotated part: every query head holds dim + rot_dim rows in ``qc``, the down-projection rot_dim more rows
+    # after the latent's; ``freqs`` fp32 [rot_dim / 2] are the pairs' angular steps per position. ``gate_col``: first
+    # row of the output gate's projection inside ``qc`` (None: no gate). Rows of ``qc`` are padded to a multiple of 8.
+    freqs: Optional[torch.Tensor] = None
+    gate_col: Optional[int] = None
 
     def tensors(self):
-        return [t for t in (self.qc, self.kv_norm, self.uk_t, self.uv, self.o) if t is not None]
+        return [t for t in (self.qc, self.kv_norm, self.uk_t, self.uv, self.o, self.freqs) if t is not None]
 
 
 @dataclass
@@ -767,9 +775,12 @@ class DecayMixWeights:
 
 @dataclass
 class DenseMLPWeights:
-    """``gu`` [2 ff, W]: gate rows, then up rows; ``down`` [W, ff]."""
+    """``gu`` [2 ff, W]: gate rows, then up rows (an ungated feed-forward: [ff, W], the up rows alone); ``down``
+    [W, ff]; ``act_params``: the activation's learned numbers in the form the kernel takes (xIELU: softplus(p),
+    1/2 + softplus(q))."""
     gu: torch.Tensor
     down: torch.Tensor
+    act_params: tuple = ()
 
     def tensors(self):
         return [self.gu, self.down]
@@ -966,3 +977,186 @@ def babotar_state_dict(cfg: ModelConfig, seed: int = 0) -> Dict[str, torch.Tenso
     """The random weights of :func:`random_babotar_weights` under their checkpoint names (bf16; tests, examples)."""
     get = _babotar_random(cfg, seed)
     return {n: get(n).to(torch.bfloat16) for n in babotar_shapes(cfg)}
+
+
+# ------------------------------------------------------------------------------ post-norm per-layer designs (Lamisun)
+@dataclass
+class DiffAttnWeights:
+    """Differential attention: ``proj`` [q | k | v rows padded to 8, W] (q: heads x 2 maps x dim, k: kv_heads x 2
+    maps x dim, v: kv_heads x vdim), ``cols`` the first row of each part; ``q_norm`` / ``k_norm`` [dim] or None;
+    ``lam``: the weight of the second map, exp(lq1 . lk1) - exp(lq2 . lk2) + diff, formed once in fp32; ``o``
+    [W, heads * vdim]."""
+    proj: torch.Tensor
+    cols: Dict[str, int]
+    q_norm: Optional[torch.Tensor]
+    k_norm: Optional[torch.Tensor]
+    lam: float
+    o: torch.Tensor
+
+    def tensors(self):
+        return [t for t in (self.proj, self.q_norm, self.k_norm, self.o) if t is not None]
+
+
+@dataclass
+class PostBlockWeights:
+    """One block with the norm on each sublayer's output: ``canon1`` / ``canon2`` [W, taps] the input convolutions of
+    the mixer and the feed-forward, ``norm1`` / ``norm2`` [W], ``dwa`` fp32 [layer + 2] the weights of the depth
+    average that leaves the layer (or None)."""
+    norm1: torch.Tensor
+    norm2: Optional[torch.Tensor]
+    canon1: Optional[torch.Tensor]
+    canon2: Optional[torch.Tensor]
+    dwa: Optional[torch.Tensor]
+    mix: object
+    mlp: Optional[DenseMLPWeights]
+
+    def tensors(self):
+        out = [self.norm1] + self.mix.tensors()
+        for t in (self.norm2, self.canon1, self.canon2, self.dwa):
+            if t is not None:
+                out.append(t)
+        if self.mlp is not None:
+            out += self.mlp.tensors()
+        return out
+
+
+def lamisun_shapes(cfg: ModelConfig) -> Dict[str, tuple]:
+    """Checkpoint tensor names of a Lamisun config and their shapes."""
+    W = cfg.hidden_size
+    out = {"embed": (cfg.vocab_size, W), "final.norm": (W,), "head": (cfg.vocab_size, W)}
+    if cfg.bigram is not None:
+        out["bigram"] = (cfg.bigram.buckets + 1, W)
+    for i, spec in enumerate(cfg.layer_specs):
+        p, m = f"l{i}.", spec.mixer
+        out[p + "norm1"] = (W,)
+        if cfg.canon_taps:
+            out[p + "canon1"] = (W, cfg.canon_taps)
+        if m.kind == "latent_attention":
+            out.update({p + "mix.q": (m.heads * (m.dim + m.rot_dim), W), p + "mix.dkv": (m.kv_rank + m.rot_dim, W),
+                        p + "mix.dkv.norm": (m.kv_rank,), p + "mix.uk": (m.heads * m.dim, m.kv_rank),
+                        p + "mix.uv": (m.heads * m.vdim, m.kv_rank), p + "mix.o": (W, m.heads * m.vdim)})
+            if m.gate:
+                out[p + "mix.g"] = (m.heads * m.vdim, W)
+        else:
+            out.update({p + "mix.q": (m.heads * 2 * m.dim, W), p + "mix.k": (m.kv_heads * 2 * m.dim, W),
+                        p + "mix.v": (m.kv_heads * m.vdim, W), p + "mix.o": (W, m.heads * m.vdim)})
+            if m.qk_norm:
+                out.update({p + "mix.q.norm": (m.dim,), p + "mix.k.norm": (m.dim,)})
+            out.update({p + "mix." + n: (m.dim,) for n in ("lq1", "lk1", "lq2", "lk2")})
+        if spec.mlp is not None:
+            out.update({p + "norm2": (W,), p + "mlp.up": (spec.mlp.ff, W), p + "mlp.down": (W, spec.mlp.ff),
+                        p + "mlp.act": (2,)})
+            if cfg.canon_taps and cfg.canon_ffn:
+                out[p + "canon2"] = (W, cfg.canon_taps)
+        if cfg.depth_average:
+            out[p + "dwa"] = (i + 2,)
+    return out
+
+
+def _lamisun_finish(cfg: ModelConfig, get, device, dtype) -> ModelWeights:
+    """``get(name)`` returns the checkpoint tensor of that name (CPU). Shapes are checked against the config. Every
+    input projection of a mixer becomes one matrix (latent attention: q | down-projection | gate; differential
+    attention: q | k | v); numbers that are fixed once the weights are known (the second map's weight, the
+    activation's two coefficients, the rotation's angular steps) are formed here, in fp32."""
+    shapes = lamisun_shapes(cfg)
+
+    def g(name):
+        t = get(name)
+        if tuple(t.shape) != shapes[name]:
+            raise ValueError(f"{name} has shape {tuple(t.shape)}, the config says {shapes[name]}")
+        return t
+
+    def dev(t, dt=dtype):
+        return None if t is None else t.to(device=device, dtype=dt).contiguous()
+
+    def f32(t):
+        return dev(t, torch.float32)
+
+    def softplus(z: float) -> float:
+        return float(torch.nn.functional.softplus(torch.tensor(z, dtype=torch.float32), threshold=80.0))
+    layers = []
+    for i, spec in enumerate(cfg.layer_specs):
+        p, m = f"l{i}.", spec.mixer
+        if m.kind == "latent_attention":
+            parts = [("q", g(p + "mix.q")), ("dkv", g(p + "mix.dkv"))]
+            if m.gate:
+                parts.append(("g", g(p + "mix.g")))
+            qc, cols = _cat_rows(parts)
+            freqs = None
+            if m.rot_dim:
+                freqs = f32(torch.tensor([m.rot.base ** (-2.0 * j / m.rot.dims) for j in range(m.rot.dims // 2)],
+                                         dtype=torch.float64))
+            mix = LatentAttnWeights(
+                qc=dev(qc), own_kv=True, kv_norm=dev(g(p + "mix.dkv.norm")),
+                uk_t=dev(_heads_t(g(p + "mix.uk"), m.heads, m.dim, m.kv_rank, i)), uv=dev(g(p + "mix.uv")),
+                o=dev(g(p + "mix.o")), freqs=freqs, gate_col=cols.get("g"))
+        else:
+            proj, cols = _cat_rows([("q", g(p + "mix.q")), ("k", g(p + "mix.k")), ("v", g(p + "mix.v"))])
+            lq1, lk1, lq2, lk2 = (g(p + "mix." + n).float() for n in ("lq1", "lk1", "lq2", "lk2"))
+            lam = float(torch.exp((lq1 * lk1).sum()) - torch.exp((lq2 * lk2).sum()) + torch.tensor(m.diff))
+            mix = DiffAttnWeights(dev(proj), cols, dev(g(p + "mix.q.norm")) if m.qk_norm else None,
+                                  dev(g(p + "mix.k.norm")) if m.qk_norm else None, lam, dev(g(p + "mix.o")))
+        mlp = None
+        if spec.mlp is not None:
+            a = g(p + "mlp.act").float()
+            mlp = DenseMLPWeights(dev(g(p + "mlp.up")), dev(g(p + "mlp.down")),
+                                  (softplus(float(a[0])), 0.5 + softplus(float(a[1]))))
+        canon = bool(cfg.canon_taps)
+        layers.append(PostBlockWeights(
+            dev(g(p + "norm1")), dev(g(p + "norm2")) if mlp is not None else None,
+            dev(g(p + "canon1")) if canon else None,
+            dev(g(p + "canon2")) if canon and cfg.canon_ffn and mlp is not None else None,
+            f32(g(p + "dwa")) if cfg.depth_average else None, mix, mlp))
+    vp = math.ceil(cfg.vocab_size / 16) * 16
+    head = torch.zeros(vp, cfg.hidden_size, dtype=dtype, device=device)
+    head[:cfg.vocab_size].copy_(g("head").to(device=device, dtype=dtype))
+    extra = {"bigram": dev(g("bigram"))} if cfg.bigram is not None else {}
+    return ModelWeights(wte=dev(g("embed")), wpe=None, layers=layers, lnf_w=dev(g("final.norm")), lnf_b=None,
+                        head=Linear(head), extra=extra)
+
+
+def load_lamisun_weights(cfg: ModelConfig, reader, device="cpu", dtype=torch.bfloat16) -> ModelWeights:
+    return _lamisun_finish(cfg, lambda n: reader.get(n), device, dtype)
+
+
+def _lamisun_random(cfg: ModelConfig, seed: int, device="cpu"):
+    import zlib
+
+    shapes = lamisun_shapes(cfg)
+
+    def get(name: str) -> torch.Tensor:
+        gen = torch.Generator(device=device)
+        gen.manual_seed((seed * 1000003 + zlib.crc32(name.encode())) & 0x7FFFFFFF)
+        shp = shapes[name]
+        t = torch.randn(*shp, generator=gen, dtype=torch.float32, device=device)
+        last = name.split(".")[-1]
+        if last.startswith("norm") or name == "final.norm":
+            t = 1.0 + 0.1 * t
+        elif last == "dwa":  # mostly the layer's own result, a little of every earlier one
+            t = 0.1 * t
+            t[-1] += 1.0
+        elif last in ("canon1", "canon2"):
+            t = t * shp[1] ** -0.5
+        elif last in ("lq1", "lk1", "lq2", "lk2"):
+            t = 0.4 * t
+        elif last == "act":
+            t = 0.5 * t
+        elif name == "embed":
+            t = t / max(cfg.embedding_scale, 1e-6)
+        elif len(shp) == 2 and name != "bigram":
+            t = t * shp[1] ** -0.5
+        return t.to(torch.bfloat16).float()
+    return get
+
+
+def random_lamisun_weights(cfg: ModelConfig, device="cpu", dtype=torch.bfloat16, seed: int = 0) -> ModelWeights:
+    """Random-init weights of a Lamisun config (values rounded to bf16, so a bf16 and an fp32 run hold the same
+    model): projections ~ N(0, 1 / fan_in), norm weights around one, depth averages around the plain stack."""
+    gen = device if torch.device(device).type == "cuda" else "cpu"  # large models: draw on the GPU
+    return _lamisun_finish(cfg, _lamisun_random(cfg, seed, gen), device, dtype)
+
+
+def lamisun_state_dict(cfg: ModelConfig, seed: int = 0) -> Dict[str, torch.Tensor]:
+    """The random weights of :func:`random_lamisun_weights` under their checkpoint names (bf16; tests, examples)."""
+    get = _lamisun_random(cfg, seed)
+    return {n: get(n).to(torch.bfloat16) for n in lamisun_shapes(cfg)}

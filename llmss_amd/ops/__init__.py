@@ -188,3 +188,12 @@ sink_attn = _route("sink_attn")
 sink_attn_mix = _route("sink_attn_mix")
 talk_mix = _route("talk_mix")
 rope_angle_table = ref.rope_angle_table
+
+# ---------------------- blocks normed on the sublayer's output / depth average / bigram embedding / differential attention
+embed_bigram = _route("embed_bigram")
+resid_norm_add = _route("resid_norm_add")
+gate_mul = _route("gate_mul")
+act_fn = _route("act_fn")
+rope_angles = _route("rope_angles")
+qk_norm_cache = _route("qk_norm_cache")
+diff_combine = _route("diff_combine")

@@ -476,12 +476,16 @@ def linear_f(x: torch.Tensor, w: torch.Tensor, out_dtype) -> torch.Tensor:
     return (x.float() @ w.float().t()).to(out_dtype)
 
 
-def head_absorb(q: torch.Tensor, uk_t: torch.Tensor, out_dtype=torch.float32) -> torch.Tensor:
-    """qa[t, h, r] = sum_d q[t, h * dim + d] * uk_t[h, r, d] -> [T, H, R] (uk_t: the key up-projection, per head
-    transposed to [R, dim])."""
+def head_absorb(q: torch.Tensor, uk_t: torch.Tensor, out_dtype=torch.float32, extra: int = 0) -> torch.Tensor:
+    """qa[t, h, r] = sum_d q[t, h * (dim + extra) + d] * uk_t[h, r, d] -> [T, H, R + extra] (uk_t: the key
+    up-projection, per head transposed to [R, dim]). ``extra`` > 0: every head of q carries that many more numbers
+    after its ``dim``, and the result that many more columns after R, left for the caller to fill."""
     H, R, dim = uk_t.shape
     T = q.shape[0]
-    return torch.einsum("thd,hrd->thr", q[:, : H * dim].float().view(T, H, dim), uk_t.float()).to(out_dtype)
+    qh = q[:, : H * (dim + extra)].float().reshape(T, H, dim + extra)[..., :dim]
+    qa = torch.zeros(T, H, R + extra, dtype=out_dtype, device=q.device)
+    qa[..., :R] = torch.einsum("thd,hrd->thr", qh, uk_t.float()).to(out_dtype)
+    return qa
 
 
 def latent_qa_dtype(cache) -> torch.dtype:
@@ -489,18 +493,44 @@ def latent_qa_dtype(cache) -> torch.dtype:
 
 
 def head_expand(o: torch.Tensor, uv: torch.Tensor, out_dtype) -> torch.Tensor:
-    """y[t, h * vd + v] = sum_r o[t, h, r] * uv[h * vd + v, r] -> [T, H * vd] in ``out_dtype``."""
-    T, H, R = o.shape
-    return torch.einsum("thr,hvr->thv", o.float(), uv.float().view(H, -1, R)).reshape(T, -1).to(out_dtype)
+    """y[t, h * vd + v] = sum_r o[t, h, r] * uv[h * vd + v, r] -> [T, H * vd] in ``out_dtype``; columns of ``o``
+    beyond uv's width are not read."""
+    T, H, _ = o.shape
+    R = uv.shape[1]
+    return torch.einsum("thr,hvr->thv", o[..., :R].float(), uv.float().view(H, -1, R)).reshape(T, -1).to(out_dtype)
+
+
+def _turn_neighbours(x: torch.Tensor, cs: torch.Tensor) -> torch.Tensor:
+    """x [T, ..., rot] with pairs (2i, 2i + 1) turned by cs [T, rot / 2, 2] = (cos, sin)."""
+    T, rot = x.shape[0], x.shape[-1]
+    shape = [T] + [1] * (x.dim() - 2) + [rot // 2]
+    c, s = cs[..., 0].view(shape), cs[..., 1].view(shape)
+    u, v = x[..., 0::2], x[..., 1::2]
+    return torch.stack([u * c - v * s, v * c + u * s], -1).reshape(x.shape)
 
 
 def latent_norm_cache(src: torch.Tensor, off: int, R: int, w: torch.Tensor, eps: float, cache: torch.Tensor,
-                      slots: torch.Tensor) -> None:
-    """cache[slot[t]] = rms_norm(src[t, off : off + R]) * w (slots < 0 are skipped); cache is [blocks, bs, R]."""
+                      slots: torch.Tensor, rot: int = 0, cs: Optional[torch.Tensor] = None,
+                      qa: Optional[torch.Tensor] = None, off_q: int = 0, qdim: int = 0) -> None:
+    """cache[slot[t], :R] = rms_norm(src[t, off : off + R]) * w (slots < 0 are skipped); cache is [blocks, bs,
+    R + rot]. ``rot`` > 0: the ``rot`` columns after the latent's are one key part shared by all heads; turned by
+    ``cs`` [T, rot / 2, 2] (neighbouring pairs) they fill the cached row, and every query head's last ``rot`` numbers
+    (head h at src[t, off_q + h * (qdim + rot) + qdim]), turned the same way, fill qa[t, h, R:]."""
     c = src[:, off:off + R].float()
     c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    if rot:
+        c = torch.cat([c, _turn_neighbours(src[:, off + R:off + R + rot].float(), cs)], -1)
+        T, H = qa.shape[0], qa.shape[1]
+        qr = src[:, off_q:off_q + H * (qdim + rot)].float().reshape(T, H, qdim + rot)[..., qdim:]
+        qa[..., R:] = _turn_neighbours(qr, cs).to(qa.dtype)
     valid = slots >= 0
-    cache.view(-1, R)[slots[valid]] = c[valid].to(cache.dtype)
+    cache.view(-1, R + rot)[slots[valid]] = c[valid].to(cache.dtype)
+
+
+def rope_angles(positions: torch.Tensor, freqs: torch.Tensor) -> torch.Tensor:
+    """fp32 [T, len(freqs), 2] = (cos, sin) of position * freqs[i], the product rounded to fp32."""
+    ang = positions.to(torch.float32)[:, None] * freqs.float()[None, :]
+    return torch.stack([torch.cos(ang), torch.sin(ang)], -1)
 
 
 def latent_attn(qa: torch.Tensor, cache: torch.Tensor, block_tables, cu_q, ctx_lens, window: int,
@@ -655,6 +685,20 @@ def gated_group_norm(o, gate, w, eps: float, act: str, c: float, out=None, out_d
     return y.to(out_dtype)
 
 
+def act_fn(x, act: str, params=()):
+    """Ungated activation of every number of x, in fp32, result in x's type. ``gelu_tanh``, ``silu``, or ``xielu``
+    with params (a, b): z > 0: a z^2 + z / 2; z <= 0: b (exp(z) - 1 - z) + z / 2."""
+    z = x.float()
+    if act == "xielu":
+        a, b = params
+        y = torch.where(z > 0, a * z * z + 0.5 * z, b * (torch.expm1(z) - z) + 0.5 * z)
+    elif act == "gelu_tanh":
+        y = torch.nn.functional.gelu(z, approximate="tanh")
+    else:
+        y = z * torch.sigmoid(z)
+    return y.to(x.dtype)
+
+
 def glu_act(gu, F_: int, act: str):
     """act(gu[:, :F]) * gu[:, F:2F]; act ``gelu_tanh`` or ``silu``."""
     g, u = gu[:, :F_].float(), gu[:, F_:2 * F_].float()
@@ -761,29 +805,39 @@ def rope_bias_cache(proj, off_q: int, off_k: int, off_v: int, bias, positions, t
 
 
 def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads: int, kv_heads: int, dim: int, vdim: int,
-              scale: float, softcap: float, all_groups: bool, max_qlen: int = 0, num_decode: int = 0):
+              scale: float, softcap: float, all_groups: bool, max_qlen: int = 0, num_decode: int = 0,
+              sink: bool = True, chunk: int = 0, vshare: int = 1):
     """Causal attention of every row over its sequence's cached keys with a sink in the softmax denominator
-    (p_j = exp(s_j) / (1 + sum exp(s))) and optionally soft-capped scores. Returns fp32 [T, heads, R]: head h's
-    weights applied to the value rows of every group side by side (``all_groups``, R = kv_heads * vdim) or of its
-    own group only (R = vdim). ``max_qlen`` (longest portion) and ``num_decode`` (leading single-row sequences) only
-    steer the choice of GPU kernel."""
+    (p_j = exp(s_j) / (1 + sum exp(s)); ``sink`` false: the ordinary softmax) and optionally soft-capped scores.
+    ``chunk`` > 0: a row at position i sees only the keys from floor(i / chunk) * chunk on. ``vshare`` > 1: that many
+    neighbouring key heads read the same value head (the value cache holds kv_heads / vshare heads). Returns fp32
+    [T, heads, R]: head h's weights applied to the value rows of every group side by side (``all_groups``,
+    R = kv_heads / vshare * vdim) or of its own group only (R = vdim). ``max_qlen`` (longest portion) and
+    ``num_decode`` (leading single-row sequences) only steer the choice of GPU kernel."""
     T = q.shape[0]
     bs = k_cache.shape[1]
     rep = heads // kv_heads
-    R = kv_heads * vdim if all_groups else vdim
+    vh = kv_heads // vshare
+    R = vh * vdim if all_groups else vdim
     out = torch.zeros(T, heads, R, dtype=torch.float32)
     for b, t0, n, p0 in _seq_rows(cu, ctx_lens):
         L = p0 + n
         blocks = block_tables[b, : -(-L // bs)].long()
         K = k_cache[blocks].reshape(-1, kv_heads, dim)[:L].float()
-        V = v_cache[blocks].reshape(-1, kv_heads, vdim)[:L].float()
+        V = v_cache[blocks].reshape(-1, vh, vdim)[:L].float().repeat_interleave(vshare, 1)
         qq = q[t0:t0 + n].view(n, heads, dim).float()
         s = torch.einsum("nhd,lhd->hnl", qq, K.repeat_interleave(rep, 1)) * scale
         if softcap:
             s = softcap * torch.tanh(s / softcap)
-        vis = torch.arange(L)[None, :] <= (p0 + torch.arange(n))[:, None]
-        e = torch.exp(s - s.amax(-1, keepdim=True).clamp(min=0)) * vis
-        p = e / (torch.exp(-s.amax(-1, keepdim=True).clamp(min=0)) + e.sum(-1, keepdim=True))
+        rows = (p0 + torch.arange(n))[:, None]
+        vis = torch.arange(L)[None, :] <= rows
+        if chunk:
+            vis = vis & (torch.arange(L)[None, :] >= rows // chunk * chunk)
+        if sink:
+            e = torch.exp(s - s.amax(-1, keepdim=True).clamp(min=0)) * vis
+            p = e / (torch.exp(-s.amax(-1, keepdim=True).clamp(min=0)) + e.sum(-1, keepdim=True))
+        else:
+            p = torch.softmax(s.masked_fill(~vis, float("-inf")), -1)
         if all_groups:
             out[t0:t0 + n] = torch.einsum("hnl,lr->nhr", p, V.reshape(L, R))
         else:
@@ -816,3 +870,77 @@ def talk_mix(O, talk, c: float, heads: int, kv_heads: int, vdim: int, out=None, 
         out.copy_(y)
         return out
     return y.to(out_dtype)
+
+
+# --------------------------------- blocks normed on the sublayer's output / depth average / bigram embedding / two maps
+def embed_bigram(ids, positions, table, scale: float, bigram, mul_prev: int, mul_cur: int, prev, cu, ctx_lens,
+                 state_slots, hist):
+    """hist[0, t] = hist[1, t] = table[ids[t]] * scale + bigram[row], row = (previous * mul_prev + ids[t] * mul_cur)
+    mod (len(bigram) - 1), or the table's last row at position 0. The token before a portion's first row is
+    prev[slot] (int64 [slots]), which is set to the portion's last token here. hist fp32 [>= 2, T, W]."""
+    buckets = bigram.shape[0] - 1
+    slots = state_slots.tolist()
+    idc = ids.clamp(0, table.shape[0] - 1)
+    before = torch.zeros_like(idc)
+    before[1:] = idc[:-1]
+    for b, t0, n, p0 in _seq_rows(cu, ctx_lens):
+        before[t0] = prev[slots[b]] if p0 > 0 else 0
+        prev[slots[b]] = idc[t0 + n - 1]
+    row = (before * mul_prev + idc * mul_cur) % buckets
+    row = torch.where(positions == 0, torch.full_like(row, buckets), row)
+    x = table[idc].float() * scale + bigram[row].float()
+    hist[0].copy_(x)
+    hist[1].copy_(x)
+
+
+def resid_norm_add(hist, n: int, y, w, eps: float, dwa=None):
+    """x = hist[n] (fp32 rows, in place) += rms_norm(y) * w. With ``dwa`` (fp32 [n + 1]) also hist[n + 1] =
+    sum_{j <= n} dwa[j] hist[j], the sum taken over the updated x. Returns the rows the next reader takes: hist[n + 1]
+    with dwa, else hist[n]."""
+    yf = y.float()
+    x = hist[n]
+    x.add_(yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * w.float())
+    if dwa is None:
+        return x
+    hist[n + 1].copy_(torch.einsum("j,jtw->tw", dwa.float(), hist[:n + 1]))
+    return hist[n + 1]
+
+
+def gate_mul(y, src, col: int):
+    """y[t, c] *= sigmoid(src[t, col + c]) in place (fp32 math)."""
+    y.copy_((y.float() * torch.sigmoid(src[:, col:col + y.shape[1]].float())).to(y.dtype))
+    return y
+
+
+def qk_norm_cache(proj, off_q: int, off_k: int, off_v: int, qw, kw, eps: float, k_cache, v_cache, slots, heads: int,
+                  kv_heads: int, maps: int, dim: int, vdim: int):
+    """From the projection rows: queries [heads, maps, dim] and keys [kv_heads, maps, dim], each vector of ``dim``
+    divided by its root mean square and multiplied by qw / kw (None: left as they are), values [kv_heads, vdim].
+    Returns q fp32 [T, kv_heads * maps * rep * dim] ordered (key head, map, query head within the group): with the
+    keys cached as kv_heads * maps heads, row-major (key head, map), query vector n reads key head n // rep. k / v go
+    into the paged caches [blocks, block_size, kv_heads * maps * dim | kv_heads * vdim] at ``slots`` (< 0: skipped)."""
+    T = proj.shape[0]
+    rep = heads // kv_heads
+    nq, nk, nv = heads * maps * dim, kv_heads * maps * dim, kv_heads * vdim
+
+    def norm(x, w):
+        if w is None:
+            return x
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    q = norm(proj[:, off_q:off_q + nq].float().reshape(T, kv_heads, rep, maps, dim), qw)
+    k = norm(proj[:, off_k:off_k + nk].float().reshape(T, kv_heads * maps, dim), kw)
+    keep = slots >= 0
+    k_cache.view(-1, nk)[slots[keep]] = k.reshape(T, nk)[keep].to(k_cache.dtype)
+    v_cache.view(-1, nv)[slots[keep]] = proj[:, off_v:off_v + nv][keep].to(v_cache.dtype)
+    return q.permute(0, 1, 3, 2, 4).reshape(T, nq).contiguous()
+
+
+def diff_combine(O, lam: float, eps: float, mult: float, heads: int, kv_heads: int, vdim: int, out_dtype):
+    """O fp32 [T, kv_heads * 2 * rep, vdim] ordered (key head, map, query head within the group) ->
+    y[t, head] = mult * rms_div(O[map 0] - lam * O[map 1]) -> [T, heads * vdim] in ``out_dtype``."""
+    T = O.shape[0]
+    rep = heads // kv_heads
+    Og = O.view(T, kv_heads, 2, rep, vdim)
+    o = Og[:, :, 0] - lam * Og[:, :, 1]
+    o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * mult
+    return o.reshape(T, heads * vdim).to(out_dtype)

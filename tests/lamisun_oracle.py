@@ -1,0 +1,153 @@
+"""Plain definition of the Lamisun design in float64: one function per mechanism, whole sequences, no cache, no
+batching, nothing shared with the product path. ``forward`` takes the raw config dictionary and a name -> tensor
+dictionary under the checkpoint's names and returns the logits of every position and the residual stream after
+every layer."""
+import math
+
+import torch
+
+F64 = torch.float64
+
+
+def rms_div(x, eps):
+    return x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+
+
+def softplus(z):
+    return math.log1p(math.exp(-abs(z))) + max(z, 0.0)
+
+
+def xielu(z, p, q):
+    """Quadratic above zero, saturating exponential below; p and q are the raw (pre-softplus) numbers."""
+    ap, aq = softplus(float(p)), 0.5 + softplus(float(q))
+    pos = ap * z * z + 0.5 * z
+    neg = aq * (torch.expm1(z) - z) + 0.5 * z
+    return torch.where(z > 0, pos, neg)
+
+
+def embed(tokens, table, bigram, scale, buckets, mul_prev, mul_cur):
+    """Token row times ``scale`` plus a hashed row of the (previous, current) pair; the first token takes the
+    table's last row."""
+    x = torch.zeros(len(tokens), table.shape[1], dtype=F64)
+    for t, tok in enumerate(tokens):
+        row = buckets if t == 0 else (int(tokens[t - 1]) * mul_prev + int(tok) * mul_cur) % buckets
+        x[t] = table[int(tok)] * scale + bigram[row]
+    return x
+
+
+def causal_conv(h, w):
+    """h [T, C], w [C, taps]; column taps - 1 multiplies the current row, column 0 the row taps - 1 back."""
+    T, C = h.shape
+    taps = w.shape[1]
+    out = torch.zeros(T, C, dtype=F64)
+    for t in range(T):
+        for j in range(taps):
+            s = t - (taps - 1) + j
+            if s >= 0:
+                out[t] += w[:, j] * h[s]
+    return out
+
+
+def rotate_pairs(x, base, dims):
+    """x [T, ..., n]: the first ``dims`` numbers of the last axis turn, neighbours (2i, 2i + 1) forming a pair that
+    turns by position * base^(-2i / dims)."""
+    T = x.shape[0]
+    out = x.clone()
+    for i in range(dims // 2):
+        ang = torch.arange(T, dtype=F64) * base ** (-2.0 * i / dims)
+        c = torch.cos(ang).view(T, *([1] * (x.dim() - 2)))
+        s = torch.sin(ang).view(T, *([1] * (x.dim() - 2)))
+        u, v = x[..., 2 * i], x[..., 2 * i + 1]
+        out[..., 2 * i] = u * c - v * s
+        out[..., 2 * i + 1] = v * c + u * s
+    return out
+
+
+def visible(T, chunk=0):
+    """[T, T] booleans: key j is seen from position i when j <= i and, with ``chunk`` > 0, both lie in the same
+    block of ``chunk`` positions counted from 0."""
+    i = torch.arange(T)[:, None]
+    j = torch.arange(T)[None, :]
+    vis = j <= i
+    if chunk:
+        vis = vis & (i // chunk == j // chunk)
+    return vis
+
+
+def softmax_rows(s, vis):
+    s = s.masked_fill(~vis, float("-inf"))
+    e = torch.exp(s - s.amax(-1, keepdim=True))
+    return e / e.sum(-1, keepdim=True)
+
+
+def latent_attention(h, m, w, eps):
+    """h [T, W]; m the mixer's config; w maps short names (q, dkv, dkv.norm, uk, uv, g, o) to tensors."""
+    T = h.shape[0]
+    H, d, r, dv, R = int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), int(m["kv_rank"])
+    base, dims = float(m["rot"]["base"]), int(m["rot"]["dims"])
+    q = (h @ w["q"].T).view(T, H, d + r)
+    q_plain, q_rot = q[..., :d], rotate_pairs(q[..., d:], base, dims)
+    down = h @ w["dkv"].T
+    c = rms_div(down[:, :R], eps) * w["dkv.norm"]
+    k_rot = rotate_pairs(down[:, R:], base, dims)  # one vector per position, shared by the heads
+    k_plain = (c @ w["uk"].T).view(T, H, d)
+    v = (c @ w["uv"].T).view(T, H, dv)
+    vis = visible(T)
+    heads = []
+    for a in range(H):
+        s = (q_plain[:, a] @ k_plain[:, a].T + q_rot[:, a] @ k_rot.T) * float(m["scale"])
+        heads.append(softmax_rows(s, vis) @ v[:, a])
+    o = torch.cat(heads, -1) * torch.sigmoid(h @ w["g"].T)
+    return o @ w["o"].T
+
+
+def diff_attention(h, m, w, eps):
+    """Two softmax maps per head over the same values, the second subtracted with one learned weight per layer;
+    h [T, W]; w maps short names (q, k, v, q.norm, k.norm, lq1, lk1, lq2, lk2, o) to tensors."""
+    T = h.shape[0]
+    H, G, d, dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
+    diff = float(m["diff"])
+    q = rms_div((h @ w["q"].T).view(T, H, 2, d), eps) * w["q.norm"]
+    k = rms_div((h @ w["k"].T).view(T, G, 2, d), eps) * w["k.norm"]
+    v = (h @ w["v"].T).view(T, G, dv)
+    lam = math.exp(float((w["lq1"] * w["lk1"]).sum())) - math.exp(float((w["lq2"] * w["lk2"]).sum())) + diff
+    vis = visible(T, int((m.get("mask") or {}).get("size") or 0))
+    heads = []
+    for a in range(H):
+        g = a // (H // G)
+        maps = [softmax_rows((q[:, a, n] @ k[:, g, n].T) * float(m["scale"]), vis) @ v[:, g] for n in range(2)]
+        heads.append(rms_div(maps[0] - lam * maps[1], eps) * (1.0 - diff))
+    return torch.cat(heads, -1) @ w["o"].T
+
+
+def feed_forward(h, w):
+    return xielu(h @ w["up"].T, w["act"][0], w["act"][1]) @ w["down"].T
+
+
+MIXERS = {"latent_attention": latent_attention, "attention": diff_attention}
+
+
+def forward(cfg, sd, tokens):
+    """(logits [T, vocab], residual after every layer [layers, T, W]) in float64."""
+    sd = {k: v.to(F64) for k, v in sd.items()}
+    eps = float(cfg["norm"]["eps"])
+    bg = cfg["embedding"]["bigram"]
+    x = embed(tokens, sd["embed"], sd["bigram"], float(cfg["embedding"]["scale"]), int(bg["buckets"]),
+              int(bg["mul_prev"]), int(bg["mul_cur"]))
+    results = [x]  # what every layer produced, the embedding first
+    after = []
+    for i, L in enumerate(cfg["layers"]):
+        p = f"l{i}."
+
+        def part(pre):
+            return {k[len(p + pre):]: v for k, v in sd.items() if k.startswith(p + pre)}
+        h = x + causal_conv(x, sd[p + "canon1"])
+        x = x + rms_div(MIXERS[L["type"]](h, L["mixer"], part("mix."), eps), eps) * sd[p + "norm1"]
+        if L.get("mlp") is not None:
+            h = x + causal_conv(x, sd[p + "canon2"])
+            x = x + rms_div(feed_forward(h, part("mlp.")), eps) * sd[p + "norm2"]
+        results.append(x)
+        x = sum(sd[p + "dwa"][j] * results[j] for j in range(i + 2))
+        after.append(x)
+    y = rms_div(x, eps) * sd["final.norm"]
+    return y @ sd["head"].T, torch.stack(after)
