@@ -18,14 +18,31 @@
 // and accumulates with lanes over the R latent dimensions (NR = ceil(R / 64) registers per lane).
 #include "anytype.h"
 
-// c = rms_norm(src[t, off : off + R]) * w, written to cache[slot[t], :] (slot < 0: not cached) in fp32 math
-template <typename T>
+// c = rms_norm(src[t, off : off + R]) * w, written to cache[slot[t], :R] (slot < 0: not cached) in fp32 math.
+// rot > 0: the cached row is [c | k_rot], k_rot = src[t, off + R : off + R + rot] with neighbouring pairs (2i, 2i + 1)
+// turned by cs[t, i] = (cos, sin); and every query head's rotated part - head h holds qdim plain numbers, then rot -
+// is turned the same way into qa[t, h, R : R + rot] (qa [T, H, R + rot] in its own type TQ).
+template <typename T, typename TQ>
 __global__ __launch_bounds__(64) void latent_norm_cache_kernel(const T* __restrict__ src, int64_t lds_, int off,
                                                                const T* __restrict__ w, float eps,
                                                                T* __restrict__ cache, const int64_t* __restrict__ slots,
-                                                               int R) {
+                                                               int R, int rot, const float* __restrict__ cs,
+                                                               TQ* __restrict__ qa, int off_q, int H, int qdim) {
   const int t = blockIdx.x, lane = threadIdx.x;
   const int64_t slot = slots[t];
+  const int half = rot >> 1;
+  const float* tab = cs + (int64_t)t * half * 2;
+  if (rot) {
+    const T* q = src + (int64_t)t * lds_ + off_q;
+    TQ* dst = qa + (int64_t)t * H * (R + rot) + R;
+    for (int e = lane; e < H * half; e += 64) {
+      const int h = e / half, i = e - h * half;
+      const T* p = q + (int64_t)h * (qdim + rot) + qdim + 2 * i;
+      const float u = El<T>::ld(p), v = El<T>::ld(p + 1), c = tab[2 * i], sn = tab[2 * i + 1];
+      El<TQ>::st(dst + (int64_t)h * (R + rot) + 2 * i, u * c - v * sn);
+      El<TQ>::st(dst + (int64_t)h * (R + rot) + 2 * i + 1, v * c + u * sn);
+    }
+  }
   if (slot < 0) return;
   const T* s = src + (int64_t)t * lds_ + off;
   float ss = 0.f;
@@ -35,15 +52,46 @@ __global__ __launch_bounds__(64) void latent_norm_cache_kernel(const T* __restri
   }
   ss = warp_sum(ss);
   const float inv = 1.0f / sqrtf(ss / (float)R + eps);
-  T* dst = cache + slot * (int64_t)R;
+  T* dst = cache + slot * (int64_t)(R + rot);
   for (int r = lane; r < R; r += 64) El<T>::st(dst + r, El<T>::ld(s + r) * inv * El<T>::ld(w + r));
+  for (int i = lane; i < half; i += 64) {
+    const float u = El<T>::ld(s + R + 2 * i), v = El<T>::ld(s + R + 2 * i + 1), c = tab[2 * i], sn = tab[2 * i + 1];
+    El<T>::st(dst + R + 2 * i, u * c - v * sn);
+    El<T>::st(dst + R + 2 * i + 1, v * c + u * sn);
+  }
 }
 
+// dq: storage type of qa (0 bf16, 1 fp32); only read when rot > 0
 void launch_latent_norm_cache(const void* src, int64_t ld, int off, const void* w, float eps, void* cache,
-                              const void* slots, int T_, int R, int dt, hipStream_t st) {
+                              const void* slots, int T_, int R, int rot, const void* cs, void* qa, int off_q, int H,
+                              int qdim, int dt, int dq, hipStream_t st) {
   if (T_ == 0) return;
-  DISPATCH_T(dt, T, (latent_norm_cache_kernel<T><<<T_, 64, 0, st>>>((const T*)src, ld, off, (const T*)w, eps,
-                                                                     (T*)cache, (const int64_t*)slots, R)));
+  if (rot < 0 || (rot & 1)) throw std::runtime_error("latent_norm_cache: the rotated part must be even");
+  DISPATCH_T(dt, T, DISPATCH_T(rot ? dq : 1, TQ, (latent_norm_cache_kernel<T, TQ><<<T_, 64, 0, st>>>(
+      (const T*)src, ld, off, (const T*)w, eps, (T*)cache, (const int64_t*)slots, R, rot, (const float*)cs, (TQ*)qa,
+      off_q, H, qdim))));
+  HIP_CHECK_LAUNCH();
+}
+
+// cs[t, i] = (cos, sin) of fl(position[t] * freqs[i]): the angle is the fp32 product, its cosine and sine are
+// evaluated in double and rounded once
+__global__ __launch_bounds__(256) void rope_angles_kernel(const int64_t* __restrict__ positions,
+                                                          const float* __restrict__ freqs, float* __restrict__ cs,
+                                                          int T_, int half) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= T_ * half) return;
+  const int t = e / half, i = e - t * half;
+  const float ang = (float)positions[t] * freqs[i];
+  double sn, c;
+  sincos((double)ang, &sn, &c);
+  cs[2 * (int64_t)e] = (float)c;
+  cs[2 * (int64_t)e + 1] = (float)sn;
+}
+
+void launch_rope_angles(const void* positions, const void* freqs, void* cs, int T_, int half, hipStream_t st) {
+  if (T_ == 0 || half == 0) return;
+  rope_angles_kernel<<<(T_ * half + 255) / 256, 256, 0, st>>>((const int64_t*)positions, (const float*)freqs,
+                                                              (float*)cs, T_, half);
   HIP_CHECK_LAUNCH();
 }
 

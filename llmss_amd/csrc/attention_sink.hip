@@ -14,6 +14,11 @@
 //
 // The sink enters the online softmax as its initial state: running maximum 0, running denominator 1, no value.
 //
+// Options that other designs use: `sink` 0 makes it the ordinary softmax (no unit in the denominator); `chunk` > 0
+// lets position i see only the keys from floor(i / chunk) * chunk on (blocks counted from position 0 of the
+// sequence); `vshare` > 1 lets that many neighbouring key heads read one value head (the value cache then holds
+// G / vshare heads) - differential attention caches the two maps of a key head as two key heads over one value head.
+//
 // One kernel serves portions of prompts, continued portions and single decoded tokens: a row finds its sequence and
 // position through cu / ctx_lens and reads every key, those of its own step too, from the paged cache.
 // Scores, softmax and sums are fp32; the cache is read in the model's storage type.
@@ -86,7 +91,7 @@ __global__ void sink_attn_kernel(const float* __restrict__ q, const T* __restric
                                  const int* __restrict__ bt, int maxb, const int* __restrict__ cu,
                                  const int* __restrict__ ctx, float* __restrict__ out, int B, int H, int G, int dim,
                                  int vdim, int bs, float scale, float cap, int all, int KB, int Dp, int hchunks,
-                                 int RVchunk) {
+                                 int RVchunk, int sink, int chunk, int vshare) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   T* tile = reinterpret_cast<T*>(smem);
   float* qs = reinterpret_cast<float*>(smem + (((size_t)KB * Dp * sizeof(T) + 15) & ~(size_t)15));
@@ -100,11 +105,12 @@ __global__ void sink_attn_kernel(const float* __restrict__ q, const T* __restric
   const int hl0 = (blockIdx.y % hchunks) * NWT;
   const bool live = hl0 + wv < rep;  // this wave scores a head
   const int h = g * rep + hl0 + wv;
-  const int RVtot = all ? G * vdim : vdim;
+  const int GV = G / vshare;  // value heads
+  const int RVtot = all ? GV * vdim : vdim;
   const int v0 = blockIdx.z * RVchunk;
   const int RV = min(RVchunk, RVtot - v0);
-  const int64_t vrow = (int64_t)G * vdim;
-  const int voff = (all ? 0 : g * vdim) + v0;
+  const int64_t vrow = (int64_t)GV * vdim;
+  const int voff = (all ? 0 : (g / vshare) * vdim) + v0;
   const int cs = NR2 * 64;  // columns per wave
   constexpr int VK = NR2 >= 4 ? 8 : 16;  // keys whose value loads are in flight together
   const RowSeq r = row_seq(cu, ctx, B, t);
@@ -124,11 +130,12 @@ __global__ void sink_attn_kernel(const float* __restrict__ q, const T* __restric
   for (int hh = 0; hh < NWT; ++hh)
 #pragma unroll
     for (int i = 0; i < NR2; ++i) acc[hh][i] = 0.f;
-  float m = 0.f, l = 1.f;  // the sink: score 0, weight exp(0 - m), no value
+  // the sink: score 0, weight exp(0 - m), no value; without it the first block of keys sets the maximum
+  float m = sink ? 0.f : -INFINITY, l = sink ? 1.f : 0.f;
   const float icap = cap > 0.f ? 1.0f / cap : 0.f;
   const int* btr = bt + (int64_t)r.b * maxb;
   const int c0 = wv * cs + lane;  // this lane's first column within the chunk
-  for (int j0 = 0; j0 <= r.pos; j0 += KB) {
+  for (int j0 = chunk > 0 ? (r.pos / chunk) * chunk : 0; j0 <= r.pos; j0 += KB) {
     const int nk = min(KB, r.pos - j0 + 1);
     __syncthreads();
     for (int kk = threadIdx.x; kk < nk; kk += blockDim.x) {
@@ -231,7 +238,7 @@ __global__ void sink_attn_kernel(const float* __restrict__ q, const T* __restric
 template <typename T>
 static void sink_attn_t(const void* q, const void* kc, const void* vc, const void* bt, int maxb, const void* cu,
                         const void* ctx, void* out, int T_, int B, int H, int G, int dim, int vdim, int bs,
-                        float scale, float cap, int all, hipStream_t st) {
+                        float scale, float cap, int all, int sink, int chunk, int vshare, hipStream_t st) {
   const int rep = H / G;
   const int NW = rep >= 8 ? 8 : (rep > 2 ? 4 : rep);  // waves = heads per workgroup: 1, 2, 4 or 8
   const int hchunks = (rep + NW - 1) / NW;
@@ -248,7 +255,7 @@ static void sink_attn_t(const void* q, const void* kc, const void* vc, const voi
   };
   while (KB > 8 && bytes(KB) > 60 * 1024) KB >>= 1;
   if (bytes(KB) > 60 * 1024) throw std::runtime_error("sink attention: head dimension too large for LDS");
-  const int RVtot = all ? G * vdim : vdim;
+  const int RVtot = all ? (G / vshare) * vdim : vdim;
   // columns per workgroup: NW waves x NR2 x 64, NR2 in {1, 2, 4} with at most 16 accumulators per lane
   int nr2 = 1;
   while (nr2 < 4 && NW * nr2 * 2 <= 16 && NW * nr2 * 64 < RVtot) nr2 <<= 1;
@@ -261,7 +268,7 @@ static void sink_attn_t(const void* q, const void* kc, const void* vc, const voi
 #define LAUNCH_SA1(NW_, NR_, WD_)                                                                            \
   sink_attn_kernel<T, NW_, NR_, WD_><<<g, NW_ * 64, bytes(KB), st>>>(                                        \
       (const float*)q, (const T*)kc, (const T*)vc, (const int*)bt, maxb, (const int*)cu, (const int*)ctx,    \
-      (float*)out, B, H, G, dim, vdim, bs, scale, cap, all, KB, Dp, hchunks, RVchunk)
+      (float*)out, B, H, G, dim, vdim, bs, scale, cap, all, KB, Dp, hchunks, RVchunk, sink, chunk, vshare)
 #define LAUNCH_SA(NW_, NR_)               \
   do {                                    \
     if (words) LAUNCH_SA1(NW_, NR_, true); \
@@ -287,11 +294,12 @@ static void sink_attn_t(const void* q, const void* kc, const void* vc, const voi
 
 void launch_sink_attn(const void* q, const void* kc, const void* vc, const void* bt, int maxb, const void* cu,
                       const void* ctx, void* out, int T_, int B, int H, int G, int dim, int vdim, int bs, float scale,
-                      float cap, int all, int dt, hipStream_t st) {
+                      float cap, int all, int sink, int chunk, int vshare, int dt, hipStream_t st) {
   if (T_ == 0 || B == 0) return;
   if (G < 1 || H % G) throw std::runtime_error("sink attention: heads must be a multiple of the key/value heads");
+  if (vshare < 1 || G % vshare || chunk < 0) throw std::runtime_error("sink attention: bad vshare / chunk");
   DISPATCH_T(dt, T, (sink_attn_t<T>(q, kc, vc, bt, maxb, cu, ctx, out, T_, B, H, G, dim, vdim, bs, scale, cap, all,
-                                    st)));
+                                    sink, chunk, vshare, st)));
   HIP_CHECK_LAUNCH();
 }
 
@@ -308,7 +316,8 @@ template <int DK, int NVT>
 __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
     const float* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
-    float* __restrict__ out, int H, int G, int GE, int vdim, int bs, float scale, float cap, int all, int nvch) {
+    float* __restrict__ out, int H, int G, int GE, int vdim, int bs, float scale, float cap, int all, int nvch,
+    int sink, int chunk, int vshare) {
   constexpr int BKV = 64;
   constexpr int LDK = DK + 16;
   constexpr int VCH = NVT * 16;
@@ -331,10 +340,12 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
   const int row = r0 + slot / GE, h = h0 + slot % GE;
   const bool valid = slot < rows_per_wg * GE && row < qlen;
   const int qpos = p0 + (valid ? row : 0);
-  const int RVtot = all ? G * vdim : vdim;
+  const int qlo = chunk > 0 ? (qpos / chunk) * chunk : 0;  // the first key this row sees
+  const int GV = G / vshare;
+  const int RVtot = all ? GV * vdim : vdim;
   const int v0 = vch * VCH;
-  const int64_t vrow = (int64_t)G * vdim;
-  const int voff = (all ? 0 : kvh * vdim) + v0;
+  const int64_t vrow = (int64_t)GV * vdim;
+  const int voff = (all ? 0 : (kvh / vshare) * vdim) + v0;
 
   s16x8 qf[DK / 32];
   {
@@ -347,11 +358,15 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
   f32x4 o[NVT];
 #pragma unroll
   for (int i = 0; i < NVT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = 0.f, lsum = 1.f;  // the sink: score 0, weight exp(0 - m), no value
+  // the sink: score 0, weight exp(0 - m), no value; without it a masked score's stand-in is the starting maximum
+  float m = sink ? 0.f : -1.0e30f, lsum = sink ? 1.f : 0.f;
   const float icap = cap > 0.f ? 1.0f / cap : 0.f;
   const int r_last = min(qlen, r0 + rows_per_wg) - 1;
   const int kv_end = p0 + r_last + 1;
+  const int kv_begin = chunk > 0 ? ((p0 + r0) / chunk) * chunk : 0;  // the first row's block starts first
   const int wave_qhi = p0 + min(qlen - 1, r0 + (16 * w + 15) / GE);
+  const int wave_first = p0 + min(qlen - 1, r0 + (16 * w) / GE);
+  const int wave_lo = chunk > 0 ? (wave_first / chunk) * chunk : 0;
   const int* bt = block_tables + (int64_t)b * max_blocks;
   constexpr int CHK = DK / 8, CHV = VCH / 8;
   // Software pipeline: the next tile's 16-byte chunks are fetched into registers while this tile is computed from
@@ -393,14 +408,15 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
   };
   // a wave none of whose slots holds a row (a single decoded row fills part of the first wave) only helps to stage
   const bool wave_rows = r0 + (16 * w) / GE < qlen && 16 * w < rows_per_wg * GE;
-  if (kv_end > 0) load_tile(0);  // (a padded row has no keys at all)
-  for (int kv0 = 0; kv0 < kv_end; kv0 += BKV) {
+  if (kv_end > kv_begin) load_tile(kv_begin);  // (a padded row has no keys at all)
+  for (int kv0 = kv_begin; kv0 < kv_end; kv0 += BKV) {
     __syncthreads();  // every wave is done reading the previous tile
     store_tile();
     __syncthreads();
     if (kv0 + BKV < kv_end) load_tile(kv0 + BKV);
     if (!wave_rows) continue;
     if (kv0 > wave_qhi) continue;  // whole tile in this wave's causal future (barriers stay uniform)
+    if (kv0 + BKV <= wave_lo) continue;  // whole tile before the block of this wave's first row
 
     f32x4 s[4];
 #pragma unroll
@@ -424,7 +440,7 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
           const float e2 = __expf(2.0f * v * icap);  // tanh(x) = 1 - 2 / (exp(2x) + 1)
           v = cap * (1.0f - 2.0f / (e2 + 1.0f));
         }
-        v = (key <= qpos && key < kv_end) ? v : -1.0e30f;
+        v = (key <= qpos && key >= qlo && key < kv_end) ? v : -1.0e30f;
         s[kt][i] = v;
         mx = fmaxf(mx, v);
       }
@@ -472,13 +488,14 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
 }
 
 // Can the matrix-core kernel take this shape? (bf16 storage is the caller's to check.)
-bool sink_attn_mfma_ok(int dim, int vdim) { return (dim == 64 || dim == 128) && vdim % 8 == 0; }
+bool sink_attn_mfma_ok(int dim, int vdim) { return (dim == 32 || dim == 64 || dim == 128) && vdim % 8 == 0; }
 
 void launch_sink_attn_mfma(const void* q, const void* kc, const void* vc, const void* bt, int maxb, const void* cu,
                            const void* ctx, void* out, int B, int max_qlen, int H, int G, int dim, int vdim, int bs,
-                           float scale, float cap, int all, hipStream_t st) {
+                           float scale, float cap, int all, int sink, int chunk, int vshare, hipStream_t st) {
   if (B == 0 || max_qlen <= 0) return;
   if (G < 1 || H % G) throw std::runtime_error("sink attention: heads must be a multiple of the key/value heads");
+  if (vshare < 1 || G % vshare || chunk < 0) throw std::runtime_error("sink attention: bad vshare / chunk");
   if (!sink_attn_mfma_ok(dim, vdim)) throw std::runtime_error("sink attention: shape not built for the matrix cores");
   const int rep = H / G;
   int GE = 1;
@@ -488,7 +505,7 @@ void launch_sink_attn_mfma(const void* q, const void* kc, const void* vc, const 
       break;
     }
   const int rows_per_wg = 64 / GE;
-  const int RVtot = all ? G * vdim : vdim;
+  const int RVtot = all ? (G / vshare) * vdim : vdim;
   const int nvt = RVtot > 128 ? 16 : (RVtot > 64 ? 8 : 4);
   const int nvch = (RVtot + nvt * 16 - 1) / (nvt * 16);
   const int64_t gy = (int64_t)G * (rep / GE) * nvch;
@@ -497,8 +514,13 @@ void launch_sink_attn_mfma(const void* q, const void* kc, const void* vc, const 
 #define LAUNCH_SAM(DK_, NVT_)                                                                                       \
   sink_attn_mfma_kernel<DK_, NVT_><<<grid, 256, 0, st>>>((const float*)q, (const bf16_t*)kc, (const bf16_t*)vc,      \
                                                          (const int*)bt, maxb, (const int*)cu, (const int*)ctx,      \
-                                                         (float*)out, H, G, GE, vdim, bs, scale, cap, all, nvch)
-  if (dim == 64) {
+                                                         (float*)out, H, G, GE, vdim, bs, scale, cap, all, nvch,     \
+                                                         sink, chunk, vshare)
+  if (dim == 32) {
+    if (nvt == 16) LAUNCH_SAM(32, 16);
+    else if (nvt == 8) LAUNCH_SAM(32, 8);
+    else LAUNCH_SAM(32, 4);
+  } else if (dim == 64) {
     if (nvt == 16) LAUNCH_SAM(64, 16);
     else if (nvt == 8) LAUNCH_SAM(64, 8);
     else LAUNCH_SAM(64, 4);
@@ -559,5 +581,97 @@ void launch_talk_mix(const void* O, const void* talk, float c, void* y, int64_t 
   if (T_ == 0) return;
   DISPATCH_T(dt, T, (talk_mix_kernel<T><<<T_, 256, 0, st>>>((const float*)O, (const float*)talk, c, (T*)y, ldy, H, G,
                                                             vdim)));
+  HIP_CHECK_LAUNCH();
+}
+
+// Queries [H, maps, dim] and keys [G, maps, dim] of a projection row, each vector of dim numbers divided by its root
+// mean square and multiplied by a weight [dim] (null: left as it is); values [G, vdim]. q -> qout fp32, ordered (key
+// head, map, query head within the group), so that with the keys cached as G * maps heads the grouped-query mapping
+// "query vector n reads key head n / rep" holds; k, v -> the paged caches at slots[t] (slot < 0: not cached).
+// One wave per vector.
+template <typename T>
+__global__ __launch_bounds__(256) void qk_norm_cache_kernel(const T* __restrict__ proj, int64_t ldp, int off_q,
+                                                            int off_k, int off_v, const T* __restrict__ qw,
+                                                            const T* __restrict__ kw, float eps,
+                                                            float* __restrict__ qout, T* __restrict__ kc,
+                                                            T* __restrict__ vc, const int64_t* __restrict__ slots,
+                                                            int H, int G, int maps, int dim, int vdim) {
+  const int t = blockIdx.x, wv = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  const T* row = proj + (int64_t)t * ldp;
+  const int64_t slot = slots[t];
+  const int rep = H / G, nqv = H * maps, nkv = G * maps;
+  for (int n = wv; n < nqv + nkv; n += nw) {
+    const bool isk = n >= nqv;
+    const int idx = isk ? n - nqv : n;
+    if (isk && slot < 0) continue;
+    const T* src = row + (isk ? off_k : off_q) + (int64_t)idx * dim;
+    const T* wt = isk ? kw : qw;
+    float inv = 1.f;
+    if (wt) {
+      float ss = 0.f;
+      for (int d = lane; d < dim; d += 64) {
+        const float v = El<T>::ld(src + d);
+        ss = fmaf(v, v, ss);
+      }
+      inv = 1.0f / sqrtf(warp_sum(ss) / (float)dim + eps);
+    }
+    if (isk) {
+      T* dst = kc + (slot * nkv + idx) * (int64_t)dim;
+      for (int d = lane; d < dim; d += 64)
+        El<T>::st(dst + d, wt ? El<T>::ld(src + d) * inv * El<T>::ld(wt + d) : El<T>::ld(src + d));
+    } else {
+      const int h = idx / maps, mp = idx - h * maps;
+      const int g = h / rep, r = h - g * rep;
+      float* dst = qout + ((int64_t)t * nqv + (g * maps + mp) * rep + r) * dim;
+      for (int d = lane; d < dim; d += 64)
+        dst[d] = wt ? El<T>::ld(src + d) * inv * El<T>::ld(wt + d) : El<T>::ld(src + d);
+    }
+  }
+  if (slot >= 0)
+    for (int e = threadIdx.x; e < G * vdim; e += blockDim.x) vc[slot * (int64_t)G * vdim + e] = row[off_v + e];
+}
+
+void launch_qk_norm_cache(const void* proj, int64_t ldp, int off_q, int off_k, int off_v, const void* qw,
+                          const void* kw, float eps, void* qout, void* kc, void* vc, const void* slots, int T_, int H,
+                          int G, int maps, int dim, int vdim, int dt, hipStream_t st) {
+  if (T_ == 0) return;
+  if (G < 1 || H % G || maps < 1) throw std::runtime_error("qk_norm_cache: heads must be a multiple of the key heads");
+  DISPATCH_T(dt, T, (qk_norm_cache_kernel<T><<<T_, 256, 0, st>>>(
+      (const T*)proj, ldp, off_q, off_k, off_v, (const T*)qw, (const T*)kw, eps, (float*)qout, (T*)kc, (T*)vc,
+      (const int64_t*)slots, H, G, maps, dim, vdim)));
+  HIP_CHECK_LAUNCH();
+}
+
+// Two maps per head, O fp32 [T, G * 2 * rep, vdim] ordered (key head, map, query head within the group):
+//   o = O[map 0] - lam * O[map 1];   y[t, head] = mult * o / sqrt(mean(o^2) + eps)      head = g * rep + r
+// One wave per (row, head).
+template <typename T>
+__global__ __launch_bounds__(256) void diff_combine_kernel(const float* __restrict__ O, float lam, float eps,
+                                                           float mult, T* __restrict__ y, int64_t ldy, int H, int G,
+                                                           int vdim) {
+  const int t = blockIdx.x, wv = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  const int rep = H / G;
+  for (int h = blockIdx.y * nw + wv; h < H; h += gridDim.y * nw) {
+    const int g = h / rep, r = h - g * rep;
+    const float* a1 = O + ((int64_t)t * 2 * H + (g * 2) * rep + r) * vdim;
+    const float* a2 = a1 + (int64_t)rep * vdim;
+    float ss = 0.f;
+    for (int c = lane; c < vdim; c += 64) {
+      const float o = a1[c] - lam * a2[c];
+      ss = fmaf(o, o, ss);
+    }
+    const float inv = mult / sqrtf(warp_sum(ss) / (float)vdim + eps);
+    T* dst = y + (int64_t)t * ldy + (int64_t)h * vdim;
+    for (int c = lane; c < vdim; c += 64) El<T>::st(dst + c, (a1[c] - lam * a2[c]) * inv);
+  }
+}
+
+void launch_diff_combine(const void* O, float lam, float eps, float mult, void* y, int64_t ldy, int T_, int H, int G,
+                         int vdim, int dt, hipStream_t st) {
+  if (T_ == 0) return;
+  if (G < 1 || H % G) throw std::runtime_error("diff_combine: heads must be a multiple of the key heads");
+  dim3 g(T_, std::min(64, (H + 3) / 4));
+  DISPATCH_T(dt, T, (diff_combine_kernel<T><<<g, 256, 0, st>>>((const float*)O, lam, eps, mult, (T*)y, ldy, H, G,
+                                                                vdim)));
   HIP_CHECK_LAUNCH();
 }

@@ -91,7 +91,9 @@ void launch_moe_gate_up_tile(const void* h, int64_t ldh, const void* wg, const v
 void launch_moe_down_tile(const void* act, const void* wd, const void* meta, void* y, int E, int maxt, int N, int F,
                           int tile_rows, hipStream_t st);
 void launch_latent_norm_cache(const void* src, int64_t ld, int off, const void* w, float eps, void* cache,
-                              const void* slots, int T_, int R, int dt, hipStream_t st);
+                              const void* slots, int T_, int R, int rot, const void* cs, void* qa, int off_q, int H,
+                              int qdim, int dt, int dq, hipStream_t st);
+void launch_rope_angles(const void* positions, const void* freqs, void* cs, int T_, int half, hipStream_t st);
 void launch_latent_attn(const void* qa, int64_t ldq, const void* cache, const void* bt, int maxb, const void* cu_q,
                         const void* ctx_lens, void* out, int64_t ldo, int T_, int B, int H, int R, int bs, int window,
                         float scale, int dt, hipStream_t st);
@@ -136,13 +138,29 @@ void launch_rope_bias_cache(const void* proj, int64_t ldp, int off_q, int off_k,
                             const void* slots, int T_, int H, int G, int dim, int vdim, int dt, hipStream_t st);
 void launch_sink_attn(const void* q, const void* kc, const void* vc, const void* bt, int maxb, const void* cu,
                       const void* ctx, void* out, int T_, int B, int H, int G, int dim, int vdim, int bs, float scale,
-                      float cap, int all, int dt, hipStream_t st);
+                      float cap, int all, int sink, int chunk, int vshare, int dt, hipStream_t st);
 bool sink_attn_mfma_ok(int dim, int vdim);
 void launch_sink_attn_mfma(const void* q, const void* kc, const void* vc, const void* bt, int maxb, const void* cu,
                            const void* ctx, void* out, int B, int max_qlen, int H, int G, int dim, int vdim, int bs,
-                           float scale, float cap, int all, hipStream_t st);
+                           float scale, float cap, int all, int sink, int chunk, int vshare, hipStream_t st);
 void launch_talk_mix(const void* O, const void* talk, float c, void* y, int64_t ldy, int T_, int H, int G, int vdim,
                      int dt, hipStream_t st);
+
+// blocks normed on the sublayer's output, depth average, bigram embedding, ungated activations, differential attention
+void launch_embed_bigram(const void* ids, const void* positions, const void* table, float scale, const void* bigram,
+                         int64_t buckets, int64_t mul_prev, int64_t mul_cur, void* prev, const void* cu,
+                         const void* ctx, const void* sslots, int B, void* h0, void* h1, int T_, int W, int vocab,
+                         int dt, hipStream_t st);
+void launch_resid_norm_add(void* hist, int64_t ldh, int n, const void* y, int64_t ldy, const void* w, float eps,
+                           const void* dwa, int T_, int W, int dt, hipStream_t st);
+void launch_gate_mul(void* y, int64_t ldy, const void* src, int64_t lds_, int T_, int N, int dt, hipStream_t st);
+void launch_act_fn(const void* x, int64_t ldx, void* out, int64_t ldo, int T_, int F, int act, float a, float b,
+                   int dt, hipStream_t st);
+void launch_qk_norm_cache(const void* proj, int64_t ldp, int off_q, int off_k, int off_v, const void* qw,
+                          const void* kw, float eps, void* qout, void* kc, void* vc, const void* slots, int T_, int H,
+                          int G, int maps, int dim, int vdim, int dt, hipStream_t st);
+void launch_diff_combine(const void* O, float lam, float eps, float mult, void* y, int64_t ldy, int T_, int H, int G,
+                         int vdim, int dt, hipStream_t st);
 
 void register_runtime(py::module_& m);  // host-side C++ runtime (runtime.cpp)
 void register_comm(py::module_& m);     // RCCL communicator (comm.cpp)
@@ -309,8 +327,13 @@ PYBIND11_MODULE(_C, m) {
     launch_moe_down_tile(CP(act), CP(wd), CP(meta), P(y), E, maxt, N, F, tile_rows, S(st));
   });
   m.def("latent_norm_cache", [](uintptr_t src, int64_t ld, int off, uintptr_t w, float eps, uintptr_t cache,
-                                uintptr_t slots, int T, int R, int dt, uintptr_t st) {
-    launch_latent_norm_cache(CP(src), ld, off, CP(w), eps, P(cache), CP(slots), T, R, dt, S(st));
+                                uintptr_t slots, int T, int R, int rot, uintptr_t cs, uintptr_t qa, int off_q, int H,
+                                int qdim, int dt, int dq, uintptr_t st) {
+    launch_latent_norm_cache(CP(src), ld, off, CP(w), eps, P(cache), CP(slots), T, R, rot, CP(cs), P(qa), off_q, H,
+                             qdim, dt, dq, S(st));
+  });
+  m.def("rope_angles", [](uintptr_t pos, uintptr_t freqs, uintptr_t cs, int T, int half, uintptr_t st) {
+    launch_rope_angles(CP(pos), CP(freqs), P(cs), T, half, S(st));
   });
   m.def("latent_attn", [](uintptr_t qa, int64_t ldq, uintptr_t cache, uintptr_t bt, int maxb, uintptr_t cu,
                           uintptr_t ctx, uintptr_t out, int64_t ldo, int T, int B, int H, int R, int bs, int window,
@@ -387,19 +410,45 @@ PYBIND11_MODULE(_C, m) {
   });
   m.def("sink_attn", [](uintptr_t q, uintptr_t kc, uintptr_t vc, uintptr_t bt, int maxb, uintptr_t cu, uintptr_t ctx,
                         uintptr_t out, int T, int B, int H, int G, int dim, int vdim, int bs, float scale, float cap,
-                        int all, int dt, uintptr_t st) {
+                        int all, int sink, int chunk, int vshare, int dt, uintptr_t st) {
     launch_sink_attn(CP(q), CP(kc), CP(vc), CP(bt), maxb, CP(cu), CP(ctx), P(out), T, B, H, G, dim, vdim, bs, scale,
-                     cap, all, dt, S(st));
+                     cap, all, sink, chunk, vshare, dt, S(st));
   });
   m.def("sink_attn_mfma_ok", &sink_attn_mfma_ok);
   m.def("sink_attn_mfma", [](uintptr_t q, uintptr_t kc, uintptr_t vc, uintptr_t bt, int maxb, uintptr_t cu,
                              uintptr_t ctx, uintptr_t out, int B, int max_qlen, int H, int G, int dim, int vdim, int bs,
-                             float scale, float cap, int all, uintptr_t st) {
+                             float scale, float cap, int all, int sink, int chunk, int vshare, uintptr_t st) {
     launch_sink_attn_mfma(CP(q), CP(kc), CP(vc), CP(bt), maxb, CP(cu), CP(ctx), P(out), B, max_qlen, H, G, dim, vdim,
-                          bs, scale, cap, all, S(st));
+                          bs, scale, cap, all, sink, chunk, vshare, S(st));
   });
   m.def("talk_mix", [](uintptr_t O, uintptr_t talk, float c, uintptr_t y, int64_t ldy, int T, int H, int G, int vdim,
                        int dt, uintptr_t st) { launch_talk_mix(CP(O), CP(talk), c, P(y), ldy, T, H, G, vdim, dt, S(st)); });
+  m.def("embed_bigram", [](uintptr_t ids, uintptr_t pos, uintptr_t table, float scale, uintptr_t bigram,
+                           int64_t buckets, int64_t mul_prev, int64_t mul_cur, uintptr_t prev, uintptr_t cu,
+                           uintptr_t ctx, uintptr_t ss, int B, uintptr_t h0, uintptr_t h1, int T, int W, int V, int dt,
+                           uintptr_t st) {
+    launch_embed_bigram(CP(ids), CP(pos), CP(table), scale, CP(bigram), buckets, mul_prev, mul_cur, P(prev), CP(cu),
+                        CP(ctx), CP(ss), B, P(h0), P(h1), T, W, V, dt, S(st));
+  });
+  m.def("resid_norm_add", [](uintptr_t hist, int64_t ldh, int n, uintptr_t y, int64_t ldy, uintptr_t w, float eps,
+                             uintptr_t dwa, int T, int W, int dt, uintptr_t st) {
+    launch_resid_norm_add(P(hist), ldh, n, CP(y), ldy, CP(w), eps, CP(dwa), T, W, dt, S(st));
+  });
+  m.def("gate_mul", [](uintptr_t y, int64_t ldy, uintptr_t src, int64_t lds_, int T, int N, int dt, uintptr_t st) {
+    launch_gate_mul(P(y), ldy, CP(src), lds_, T, N, dt, S(st));
+  });
+  m.def("act_fn", [](uintptr_t x, int64_t ldx, uintptr_t out, int64_t ldo, int T, int F, int act, float a, float b,
+                     int dt, uintptr_t st) { launch_act_fn(CP(x), ldx, P(out), ldo, T, F, act, a, b, dt, S(st)); });
+  m.def("qk_norm_cache", [](uintptr_t proj, int64_t ldp, int off_q, int off_k, int off_v, uintptr_t qw, uintptr_t kw,
+                            float eps, uintptr_t qout, uintptr_t kc, uintptr_t vc, uintptr_t slots, int T, int H, int G,
+                            int maps, int dim, int vdim, int dt, uintptr_t st) {
+    launch_qk_norm_cache(CP(proj), ldp, off_q, off_k, off_v, CP(qw), CP(kw), eps, P(qout), P(kc), P(vc), CP(slots), T,
+                         H, G, maps, dim, vdim, dt, S(st));
+  });
+  m.def("diff_combine", [](uintptr_t O, float lam, float eps, float mult, uintptr_t y, int64_t ldy, int T, int H, int G,
+                           int vdim, int dt, uintptr_t st) {
+    launch_diff_combine(CP(O), lam, eps, mult, P(y), ldy, T, H, G, vdim, dt, S(st));
+  });
   register_runtime(m);
   register_comm(m);
   register_ctrl(m);

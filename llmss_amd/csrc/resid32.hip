@@ -5,6 +5,7 @@
 // 32-bit use these kernels instead: the stream x [T, H] is fp32 and updated in place, only the normed output that
 // feeds the matrix products is rounded to the model's storage type.
 #include "anytype.h"
+#include "seqrows.h"
 
 // x[t, :] = table[ids[t], :] * scale
 template <typename T>
@@ -177,5 +178,156 @@ void launch_resid_add_norm(void* x, const void* a, int64_t lda, const void* b, i
     if (vec) resid_add_norm_kernel<T, 4><<<T_, 256, 0, st>>>(p);
     else resid_add_norm_kernel<T, 1><<<T_, 256, 0, st>>>(p);
   });
+  HIP_CHECK_LAUNCH();
+}
+
+// ---- blocks whose norm sits on the sublayer's output, results of the layers averaged over depth, bigram embedding
+//
+// The layers' results live in hist [slots, T, W] fp32 (slot stride ldh). Layer i works in place on hist[i + 1], which
+// the step before has filled with the layer's input.
+
+// hist[0][t] = hist[1][t] = table[ids[t]] * scale + bigram[row],
+//   row = (before * mul_prev + ids[t] * mul_cur) mod buckets, or `buckets` (the table's last row) at position 0.
+// `before` is the row above inside a portion and prev[slot] for a portion's first row; that workgroup then sets
+// prev[slot] to the portion's last token (it has read the old value: one workgroup, a barrier in between).
+template <typename T>
+__global__ __launch_bounds__(256) void embed_bigram_kernel(const int64_t* __restrict__ ids,
+                                                           const int64_t* __restrict__ positions,
+                                                           const T* __restrict__ table, float scale,
+                                                           const T* __restrict__ bigram, int64_t buckets,
+                                                           int64_t mul_prev, int64_t mul_cur, int64_t* __restrict__ prev,
+                                                           const int* __restrict__ cu, const int* __restrict__ ctx,
+                                                           const int* __restrict__ sslots, int B,
+                                                           float* __restrict__ h0, float* __restrict__ h1, int W,
+                                                           int vocab) {
+  const int t = blockIdx.x;
+  const RowSeq r = row_seq(cu, ctx, B, t);
+  float* d0 = h0 + (int64_t)t * W;
+  float* d1 = h1 + (int64_t)t * W;
+  if (r.pos < 0) {  // a padded row
+    for (int c = threadIdx.x; c < W; c += blockDim.x) d0[c] = d1[c] = 0.f;
+    return;
+  }
+  auto clampv = [&](int64_t id) { return id < 0 ? (int64_t)0 : (id >= vocab ? (int64_t)vocab - 1 : id); };
+  const int64_t id = clampv(ids[t]);
+  const int slot = sslots[r.b];
+  int64_t before = 0;
+  if (r.j > 0) before = clampv(ids[t - 1]);
+  else if (r.pos > 0 && slot >= 0) before = prev[slot];
+  int64_t row = (before * mul_prev + id * mul_cur) % buckets;
+  if (row < 0) row += buckets;
+  if (positions[t] == 0) row = buckets;
+  if (r.j == 0 && slot >= 0) {
+    __syncthreads();  // every thread holds the old value
+    if (threadIdx.x == 0) prev[slot] = clampv(ids[t + r.qlen - 1]);
+  }
+  const T* src = table + id * (int64_t)W;
+  const T* bg = bigram + row * (int64_t)W;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    const float v = fmaf(El<T>::ld(src + c), scale, El<T>::ld(bg + c));
+    d0[c] = v;
+    d1[c] = v;
+  }
+}
+
+void launch_embed_bigram(const void* ids, const void* positions, const void* table, float scale, const void* bigram,
+                         int64_t buckets, int64_t mul_prev, int64_t mul_cur, void* prev, const void* cu,
+                         const void* ctx, const void* sslots, int B, void* h0, void* h1, int T_, int W, int vocab,
+                         int dt, hipStream_t st) {
+  if (T_ == 0) return;
+  if (buckets < 1) throw std::runtime_error("embed_bigram: at least one bucket");
+  DISPATCH_T(dt, T, (embed_bigram_kernel<T><<<T_, 256, 0, st>>>(
+      (const int64_t*)ids, (const int64_t*)positions, (const T*)table, scale, (const T*)bigram, buckets, mul_prev,
+      mul_cur, (int64_t*)prev, (const int*)cu, (const int*)ctx, (const int*)sslots, B, (float*)h0, (float*)h1, W,
+      vocab)));
+  HIP_CHECK_LAUNCH();
+}
+
+// x = hist[n][t] += y[t] / sqrt(mean(y[t]^2) + eps) * w; with dwa also hist[n + 1][t] = sum_{j <= n} dwa[j] hist[j][t]
+// (over the updated x). The mean square is summed in fp32 from y in the storage type.
+template <typename T, int V>
+__global__ __launch_bounds__(256) void resid_norm_add_kernel(float* __restrict__ hist, int64_t ldh, int n,
+                                                             const T* __restrict__ y, int64_t ldy,
+                                                             const T* __restrict__ w, float eps,
+                                                             const float* __restrict__ dwa, int W) {
+  __shared__ float red[16];
+  const int t = blockIdx.x;
+  const T* yr = y + (int64_t)t * ldy;
+  float ss = 0.f;
+  for (int c = threadIdx.x * V; c < W; c += blockDim.x * V) {
+    if constexpr (V == 4) {
+      const f32x4 q = ld4<T>(yr + c);
+      ss += q[0] * q[0] + q[1] * q[1] + q[2] * q[2] + q[3] * q[3];
+    } else {
+      const float q = El<T>::ld(yr + c);
+      ss += q * q;
+    }
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)W + eps);
+  float* xr = hist + (int64_t)n * ldh + (int64_t)t * W;
+  float* nx = xr + ldh;
+  const float wn = dwa ? dwa[n] : 0.f;
+  for (int c = threadIdx.x * V; c < W; c += blockDim.x * V) {
+    if constexpr (V == 4) {
+      const f32x4 q = ld4<T>(yr + c), wv = ld4<T>(w + c);
+      f32x4 x = *reinterpret_cast<const f32x4*>(xr + c);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[i] += q[i] * inv * wv[i];
+      *reinterpret_cast<f32x4*>(xr + c) = x;
+      if (dwa) {
+        f32x4 a = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < n; ++j) {
+          const float wj = dwa[j];
+          const f32x4 e = *reinterpret_cast<const f32x4*>(hist + (int64_t)j * ldh + (int64_t)t * W + c);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) a[i] = fmaf(wj, e[i], a[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) a[i] = fmaf(wn, x[i], a[i]);
+        *reinterpret_cast<f32x4*>(nx + c) = a;
+      }
+    } else {
+      const float x = xr[c] + El<T>::ld(yr + c) * inv * El<T>::ld(w + c);
+      xr[c] = x;
+      if (dwa) {
+        float a = 0.f;
+        for (int j = 0; j < n; ++j) a = fmaf(dwa[j], hist[(int64_t)j * ldh + (int64_t)t * W + c], a);
+        nx[c] = fmaf(wn, x, a);
+      }
+    }
+  }
+}
+
+void launch_resid_norm_add(void* hist, int64_t ldh, int n, const void* y, int64_t ldy, const void* w, float eps,
+                           const void* dwa, int T_, int W, int dt, hipStream_t st) {
+  if (T_ == 0) return;
+  const int es = dt == 0 ? 2 : 4;
+  const bool vec = W % 4 == 0 && ldh % 4 == 0 && ((uintptr_t)hist % 16) == 0 && ((uintptr_t)y % (4 * es)) == 0 &&
+                   (ldy * es) % (4 * es) == 0 && ((uintptr_t)w % (4 * es)) == 0;
+  DISPATCH_T(dt, T, {
+    if (vec) resid_norm_add_kernel<T, 4><<<T_, 256, 0, st>>>((float*)hist, ldh, n, (const T*)y, ldy, (const T*)w, eps,
+                                                             (const float*)dwa, W);
+    else resid_norm_add_kernel<T, 1><<<T_, 256, 0, st>>>((float*)hist, ldh, n, (const T*)y, ldy, (const T*)w, eps,
+                                                         (const float*)dwa, W);
+  });
+  HIP_CHECK_LAUNCH();
+}
+
+// y[t, c] *= sigmoid(src[t, col + c])
+template <typename T>
+__global__ __launch_bounds__(256) void gate_mul_kernel(T* __restrict__ y, int64_t ldy, const T* __restrict__ src,
+                                                       int64_t lds_, int N) {
+  const int t = blockIdx.x;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < N; c += gridDim.y * blockDim.x) {
+    const float g = El<T>::ld(src + (int64_t)t * lds_ + c);
+    T* p = y + (int64_t)t * ldy + c;
+    El<T>::st(p, El<T>::ld(p) / (1.0f + expf(-g)));
+  }
+}
+
+void launch_gate_mul(void* y, int64_t ldy, const void* src, int64_t lds_, int T_, int N, int dt, hipStream_t st) {
+  if (T_ == 0 || N == 0) return;
+  dim3 g(T_, std::min(64, (N + 255) / 256));
+  DISPATCH_T(dt, T, (gate_mul_kernel<T><<<g, 256, 0, st>>>((T*)y, ldy, (const T*)src, lds_, N)));
   HIP_CHECK_LAUNCH();
 }

@@ -270,3 +270,27 @@ void launch_glu_act(const void* gu, int64_t ldg, void* out, int64_t ldo, int T_,
   DISPATCH_T(dt, T, (glu_act_kernel<T><<<g, 256, 0, st>>>((const T*)gu, ldg, (T*)out, ldo, F, act)));
   HIP_CHECK_LAUNCH();
 }
+
+// out[t, f] = act(x[t, f]), no gate. act 0: tanh-form GELU, 1: SiLU, 2: xIELU with the two coefficients (a, b):
+//   z > 0: a z^2 + z / 2;   z <= 0: b (exp(z) - 1 - z) + z / 2
+template <typename T>
+__global__ __launch_bounds__(256) void act_fn_kernel(const T* __restrict__ x, int64_t ldx, T* __restrict__ out,
+                                                     int64_t ldo, int F, int act, float a, float b) {
+  const int t = blockIdx.x;
+  for (int f = blockIdx.y * blockDim.x + threadIdx.x; f < F; f += gridDim.y * blockDim.x) {
+    const float z = El<T>::ld(x + (int64_t)t * ldx + f);
+    float y;
+    if (act == 0) y = 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    else if (act == 1) y = z / (1.0f + expf(-z));
+    else y = z > 0.f ? fmaf(a * z, z, 0.5f * z) : fmaf(b, expm1f(z) - z, 0.5f * z);
+    El<T>::st(out + (int64_t)t * ldo + f, y);
+  }
+}
+
+void launch_act_fn(const void* x, int64_t ldx, void* out, int64_t ldo, int T_, int F, int act, float a, float b,
+                   int dt, hipStream_t st) {
+  if (T_ == 0 || F == 0) return;
+  dim3 g(T_, std::min(64, (F + 255) / 256));
+  DISPATCH_T(dt, T, (act_fn_kernel<T><<<g, 256, 0, st>>>((const T*)x, ldx, (T*)out, ldo, F, act, a, b)));
+  HIP_CHECK_LAUNCH();
+}

@@ -896,42 +896,64 @@ def linear_f(x, w, out_dtype):
     return gemm_any(x, w, y, M, N, K, 1, 0, x.stride(0), 0, K, 1, 0, N)
 
 
-def head_absorb(q, uk_t, out_dtype=torch.float32):
+def head_absorb(q, uk_t, out_dtype=torch.float32, extra=0):
     H, R, dim = uk_t.shape
     T = q.shape[0]
     _rows(q, "q")
-    _check(q.shape[1] >= H * dim, "q too narrow")
+    _check(extra >= 0 and q.shape[1] >= H * (dim + extra), "q too narrow")
     _check(uk_t.is_contiguous() and uk_t.dtype == q.dtype and uk_t.is_cuda, "uk_t [H, R, dim] in q's storage type")
-    qa = torch.empty(T, H, R, dtype=out_dtype, device=q.device)
+    Rt = R + extra
+    qa = torch.empty(T, H, Rt, dtype=out_dtype, device=q.device)
     if T:
-        # batch = head: A(t, d) = q[t, h * dim + d]; B(r, d) = uk_t[h, r, d]
-        gemm_any(q, uk_t, qa, T, R, dim, H, dim, q.stride(0), R * dim, dim, 1, R, H * R)
+        # batch = head: A(t, d) = q[t, h * (dim + extra) + d]; B(r, d) = uk_t[h, r, d]; C(t, r) = qa[t, h, r]
+        gemm_any(q, uk_t, qa, T, R, dim, H, dim + extra, q.stride(0), R * dim, dim, 1, Rt, H * Rt)
     return qa
 
 
 def head_expand(o, uv, out_dtype):
-    T, H, R = o.shape
-    _check(o.is_contiguous() and o.dtype in _DT and o.is_cuda, "o [T, H, R] contiguous")
+    T, H, Rt = o.shape
+    R = uv.shape[1]
+    _check(o.is_contiguous() and o.dtype in _DT and o.is_cuda and R <= Rt, "o [T, H, >= R] contiguous")
     _rows(uv, "uv", R)
     _check(uv.is_contiguous() and uv.shape[0] % H == 0, "uv [H * vdim, R]")
     vd = uv.shape[0] // H
     y = torch.empty(T, H * vd, dtype=out_dtype, device=o.device)
     if T:
-        # batch = head: A(t, r) = o[t, h, r]; B(v, r) = uv[h * vd + v, r]; C(t, v) = y[t, h * vd + v]
-        gemm_any(o, uv, y, T, vd, R, H, R, H * R, vd * R, R, 1, vd, H * vd)
+        # batch = head: A(t, r) = o[t, h, r], r < R; B(v, r) = uv[h * vd + v, r]; C(t, v) = y[t, h * vd + v]
+        gemm_any(o, uv, y, T, vd, R, H, Rt, H * Rt, vd * R, R, 1, vd, H * vd)
     return y
 
 
-def latent_norm_cache(src, off, R, w, eps, cache, slots):
+def latent_norm_cache(src, off, R, w, eps, cache, slots, rot=0, cs=None, qa=None, off_q=0, qdim=0):
     T = src.shape[0]
     _rows(src, "src")
-    _check(0 <= off and off + R <= src.shape[1], "latent columns outside src")
-    _check(cache.dtype == src.dtype and cache.is_contiguous() and cache.dim() == 3 and cache.shape[2] == R,
-           "latent cache [blocks, block_size, R] in the model's storage type")
+    rot = int(rot)
+    _check(0 <= off and off + R + rot <= src.shape[1], "latent columns outside src")
+    _check(cache.dtype == src.dtype and cache.is_contiguous() and cache.dim() == 3 and cache.shape[2] == R + rot,
+           "latent cache [blocks, block_size, R + rot] in the model's storage type")
     _check(w.dtype == src.dtype and w.is_contiguous() and w.numel() == R, "latent norm weight")
     _check(slots.dtype == torch.int64 and slots.is_contiguous() and slots.numel() == T and slots.is_cuda, "slots")
+    H = dq = 0
+    if rot:
+        _check(rot % 2 == 0, "the rotated part must be even")
+        _f32c(cs, "angles")
+        _check(tuple(cs.shape) == (T, rot // 2, 2), "angles [T, rot / 2, 2]")
+        _check(qa.is_contiguous() and qa.is_cuda and qa.dim() == 3 and qa.shape[0] == T and qa.shape[2] == R + rot,
+               "qa [T, H, R + rot] contiguous")
+        H, dq = qa.shape[1], _dt(qa, "qa")
+        _check(off_q >= 0 and off_q + H * (qdim + rot) <= src.shape[1], "query columns outside src")
     lib().latent_norm_cache(src.data_ptr(), src.stride(0), int(off), w.data_ptr(), float(eps), cache.data_ptr(),
-                            slots.data_ptr(), T, R, _dt(src, "src"), _stream())
+                            slots.data_ptr(), T, R, rot, _ptr(cs) if rot else 0, _ptr(qa) if rot else 0, int(off_q), H,
+                            int(qdim), _dt(src, "src"), dq, _stream())
+
+
+def rope_angles(positions, freqs):
+    T = positions.numel()
+    _check(positions.dtype == torch.int64 and positions.is_contiguous() and positions.is_cuda, "positions: int64 cuda")
+    _f32c(freqs, "freqs")
+    cs = torch.empty(T, freqs.numel(), 2, dtype=torch.float32, device=positions.device)
+    lib().rope_angles(positions.data_ptr(), freqs.data_ptr(), cs.data_ptr(), T, freqs.numel(), _stream())
+    return cs
 
 
 LATENT_MFMA_RANKS = (64, 128, 256)  # latent ranks the MFMA extend kernel is built for (csrc/attention_extend.hip)
@@ -1269,7 +1291,7 @@ _SINK_MFMA = os.environ.get("LLMSS_SINK_MFMA", "1") != "0"  # 0: every shape on 
 
 
 def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, dim, vdim, scale, softcap,
-              all_groups, max_qlen=0, num_decode=0):
+              all_groups, max_qlen=0, num_decode=0, sink=True, chunk=0, vshare=1):
     """``max_qlen`` (the longest portion of the step, known on the host) > 0: a bf16 cache of a shape the matrix-core
     kernel is built for runs on it, the ``num_decode`` leading single-row sequences in one launch and the portions
     in another; everything else runs the vector kernel."""
@@ -1281,16 +1303,19 @@ def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, 
     _i32(ctx_lens, "ctx_lens", B)
     _i32(block_tables, "block_tables")
     _check(block_tables.dim() == 2 and block_tables.shape[0] >= B, "block tables [B, blocks]")
+    _check(vshare >= 1 and kv_heads % vshare == 0 and chunk >= 0, "vshare must divide the key heads")
+    vh = kv_heads // vshare
     _check(k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == v_cache.dtype
-           and k_cache.dim() == 3 and k_cache.shape[2] == kv_heads * dim and v_cache.shape[2] == kv_heads * vdim
+           and k_cache.dim() == 3 and k_cache.shape[2] == kv_heads * dim and v_cache.shape[2] == vh * vdim
            and k_cache.shape[:2] == v_cache.shape[:2], "k / v cache [blocks, block_size, kv_heads * dim | vdim]")
-    R = kv_heads * vdim if all_groups else vdim
+    R = vh * vdim if all_groups else vdim
     out = torch.empty(T, heads, R, dtype=torch.float32, device=q.device)
     nd = int(num_decode)
     _check(0 <= nd <= B, "num_decode outside the step")
     mfma = (k_cache.dtype == torch.bfloat16 and max_qlen > 0 and lib().sink_attn_mfma_ok(dim, vdim)
             and k_cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0 and _SINK_MFMA)
-    common = (heads, kv_heads, dim, vdim, k_cache.shape[1], float(scale), float(softcap or 0.0), int(bool(all_groups)))
+    common = (heads, kv_heads, dim, vdim, k_cache.shape[1], float(scale), float(softcap or 0.0), int(bool(all_groups)),
+              int(bool(sink)), int(chunk), int(vshare))
     if mfma:
         # the leading single-row sequences get a grid of their own (one row block each): in the portions' grid every
         # one of them would launch a whole prompt's worth of workgroups that exit at once, and those are not free
@@ -1332,3 +1357,89 @@ def talk_mix(O, talk, c, heads, kv_heads, vdim, out=None, out_dtype=None):
     lib().talk_mix(O.data_ptr(), _ptr(talk), float(c), out.data_ptr(), out.stride(0), T, heads, kv_heads, vdim,
                    _dt(out, "out"), _stream())
     return out
+
+
+# ---------------------- blocks normed on the sublayer's output / depth average / bigram embedding / differential attention
+def embed_bigram(ids, positions, table, scale, bigram, mul_prev, mul_cur, prev, cu, ctx_lens, state_slots, hist):
+    T = ids.numel()
+    V, W = table.shape
+    for t, nm in ((ids, "ids"), (positions, "positions")):
+        _check(t.dtype == torch.int64 and t.is_contiguous() and t.is_cuda and t.numel() == T, f"{nm}: int64 [T] cuda")
+    _check(table.is_contiguous() and bigram.is_contiguous() and bigram.dtype == table.dtype and bigram.dim() == 2
+           and bigram.shape[1] == W and bigram.shape[0] >= 2, "bigram table [buckets + 1, W] in the table's type")
+    _check(prev.dtype == torch.int64 and prev.is_contiguous() and prev.is_cuda, "prev: int64 [slots] cuda")
+    B = cu.numel() - 1
+    _i32(cu, "cu")
+    _i32(ctx_lens, "ctx_lens", B)
+    _i32(state_slots, "state_slots", B)
+    _check(hist.dtype == torch.float32 and hist.is_contiguous() and hist.dim() == 3 and hist.shape[0] >= 2
+           and tuple(hist.shape[1:]) == (T, W) and hist.is_cuda, "hist fp32 [>= 2, T, W]")
+    lib().embed_bigram(ids.data_ptr(), positions.data_ptr(), table.data_ptr(), float(scale), bigram.data_ptr(),
+                       bigram.shape[0] - 1, int(mul_prev), int(mul_cur), prev.data_ptr(), cu.data_ptr(),
+                       ctx_lens.data_ptr(), state_slots.data_ptr(), B, hist[0].data_ptr(), hist[1].data_ptr(), T, W, V,
+                       _dt(table, "table"), _stream())
+
+
+def resid_norm_add(hist, n, y, w, eps, dwa=None):
+    S, T, W = hist.shape
+    _check(hist.dtype == torch.float32 and hist.is_contiguous() and hist.is_cuda, "hist fp32 [slots, T, W]")
+    _check(0 <= n < S - (1 if dwa is not None else 0), "hist slot outside the buffer")
+    _rows(y, "y", W)
+    _check(y.shape[0] == T and w.dtype == y.dtype and w.is_contiguous() and w.numel() == W, "y rows / norm weight")
+    if dwa is not None:
+        _f32c(dwa, "dwa")
+        _check(dwa.numel() == n + 1, "dwa [n + 1]")
+    lib().resid_norm_add(hist.data_ptr(), T * W, int(n), y.data_ptr(), y.stride(0), w.data_ptr(), float(eps),
+                         _ptr(dwa), T, W, _dt(y, "y"), _stream())
+    return hist[n + 1] if dwa is not None else hist[n]
+
+
+def gate_mul(y, src, col):
+    T, N = y.shape
+    _rows(y, "y")
+    _rows(src, "src")
+    _check(src.dtype == y.dtype and src.shape[0] == T and 0 <= col and col + N <= src.shape[1], "gate columns")
+    lib().gate_mul(y.data_ptr(), y.stride(0), src.data_ptr() + col * src.element_size(), src.stride(0), T, N,
+                   _dt(y, "y"), _stream())
+    return y
+
+
+def act_fn(x, act, params=()):
+    T, F = x.shape
+    _rows(x, "x")
+    out = torch.empty(T, F, dtype=x.dtype, device=x.device)
+    a, b = (float(params[0]), float(params[1])) if act == "xielu" else (0.0, 0.0)
+    lib().act_fn(x.data_ptr(), x.stride(0), out.data_ptr(), F, T, F, {"gelu_tanh": 0, "silu": 1, "xielu": 2}[act], a, b,
+                 _dt(x, "x"), _stream())
+    return out
+
+
+def qk_norm_cache(proj, off_q, off_k, off_v, qw, kw, eps, k_cache, v_cache, slots, heads, kv_heads, maps, dim, vdim):
+    T = proj.shape[0]
+    _rows(proj, "proj")
+    nq, nk, nv = heads * maps * dim, kv_heads * maps * dim, kv_heads * vdim
+    _check(min(off_q, off_k, off_v) >= 0 and max(off_q + nq, off_k + nk, off_v + nv) <= proj.shape[1],
+           "q / k / v columns outside the projection")
+    for w_, nm in ((qw, "q norm"), (kw, "k norm")):
+        if w_ is not None:
+            _check(w_.dtype == proj.dtype and w_.is_contiguous() and w_.numel() == dim and w_.is_cuda, f"{nm} [dim]")
+    for c, n, nm in ((k_cache, nk, "k cache"), (v_cache, nv, "v cache")):
+        _check(c.dtype == proj.dtype and c.is_contiguous() and c.dim() == 3 and c.shape[2] == n,
+               f"{nm} [blocks, block_size, {n}] in the model's storage type")
+    _check(slots.dtype == torch.int64 and slots.is_contiguous() and slots.is_cuda and slots.numel() == T, "slots")
+    q = torch.empty(T, nq, dtype=torch.float32, device=proj.device)
+    lib().qk_norm_cache(proj.data_ptr(), proj.stride(0), int(off_q), int(off_k), int(off_v), _ptr(qw), _ptr(kw),
+                        float(eps), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), slots.data_ptr(), T, heads,
+                        kv_heads, maps, dim, vdim, _dt(proj, "proj"), _stream())
+    return q
+
+
+def diff_combine(O, lam, eps, mult, heads, kv_heads, vdim, out_dtype):
+    T = O.shape[0]
+    _check(O.dtype == torch.float32 and O.is_contiguous() and tuple(O.shape[1:]) == (2 * heads, vdim) and O.is_cuda,
+           "O fp32 [T, 2 * heads, vdim]")
+    _check(out_dtype in _DT, "out dtype bf16 / fp32")
+    y = torch.empty(T, heads * vdim, dtype=out_dtype, device=O.device)
+    lib().diff_combine(O.data_ptr(), float(lam), float(eps), float(mult), y.data_ptr(), y.stride(0), T, heads,
+                       kv_heads, vdim, _DT[out_dtype], _stream())
+    return y
