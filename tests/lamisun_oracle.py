@@ -80,25 +80,49 @@ def softmax_rows(s, vis):
     return e / e.sum(-1, keepdim=True)
 
 
-def latent_attention(h, m, w, eps):
-    """h [T, W]; m the mixer's config; w maps short names (q, dkv, dkv.norm, uk, uv, g, o) to tensors."""
-    T = h.shape[0]
-    H, d, r, dv, R = int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), int(m["kv_rank"])
-    base, dims = float(m["rot"]["base"]), int(m["rot"]["dims"])
-    q = (h @ w["q"].T).view(T, H, d + r)
-    q_plain, q_rot = q[..., :d], rotate_pairs(q[..., d:], base, dims)
-    down = h @ w["dkv"].T
-    c = rms_div(down[:, :R], eps) * w["dkv.norm"]
-    k_rot = rotate_pairs(down[:, R:], base, dims)  # one vector per position, shared by the heads
-    k_plain = (c @ w["uk"].T).view(T, H, d)
-    v = (c @ w["uv"].T).view(T, H, dv)
+def latent_heads(q, down, norm_w, uk, uv, H, d, r, dv, R, base, scale, eps):
+    """q [T, H * (d + r)] (per head: d plain numbers, then r that turn with the position), down [T, R + r] (the
+    latent before its norm, then one turning key part for all heads). Returns the heads' outputs [T, H * dv]."""
+    T = q.shape[0]
+    q = q.view(T, H, d + r)
+    q_plain, q_rot = q[..., :d], rotate_pairs(q[..., d:], base, r)
+    c = rms_div(down[:, :R], eps) * norm_w
+    k_rot = rotate_pairs(down[:, R:], base, r)
+    k_plain = (c @ uk.T).view(T, H, d)
+    v = (c @ uv.T).view(T, H, dv)
     vis = visible(T)
     heads = []
     for a in range(H):
-        s = (q_plain[:, a] @ k_plain[:, a].T + q_rot[:, a] @ k_rot.T) * float(m["scale"])
+        s = (q_plain[:, a] @ k_plain[:, a].T + q_rot[:, a] @ k_rot.T) * scale
         heads.append(softmax_rows(s, vis) @ v[:, a])
-    o = torch.cat(heads, -1) * torch.sigmoid(h @ w["g"].T)
-    return o @ w["o"].T
+    return torch.cat(heads, -1)
+
+
+def latent_attention(h, m, w, eps):
+    """h [T, W]; m the mixer's config; w maps short names (q, dkv, dkv.norm, uk, uv, g, o) to tensors."""
+    H, d, r, dv, R = int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), int(m["kv_rank"])
+    assert int(m["rot"]["dims"]) == r
+    o = latent_heads(h @ w["q"].T, h @ w["dkv"].T, w["dkv.norm"], w["uk"], w["uv"], H, d, r, dv, R,
+                     float(m["rot"]["base"]), float(m["scale"]), eps)
+    return (o * torch.sigmoid(h @ w["g"].T)) @ w["o"].T
+
+
+def two_map_heads(q, k, v, scale, lam, mult, chunk, eps):
+    """q [T, H, 2, d], k [T, G, 2, d] (already normed), v [T, G, dv]: per head two softmax maps over the same values,
+    o = map 0 - lam * map 1, divided by its root mean square, times mult. Returns [T, H * dv]."""
+    T, H = q.shape[0], q.shape[1]
+    G = k.shape[1]
+    vis = visible(T, chunk)
+    heads = []
+    for a in range(H):
+        g = a // (H // G)
+        maps = [softmax_rows((q[:, a, n] @ k[:, g, n].T) * scale, vis) @ v[:, g] for n in range(2)]
+        heads.append(rms_div(maps[0] - lam * maps[1], eps) * mult)
+    return torch.cat(heads, -1)
+
+
+def second_map_weight(lq1, lk1, lq2, lk2, diff):
+    return math.exp(float((lq1 * lk1).sum())) - math.exp(float((lq2 * lk2).sum())) + diff
 
 
 def diff_attention(h, m, w, eps):
@@ -110,14 +134,9 @@ def diff_attention(h, m, w, eps):
     q = rms_div((h @ w["q"].T).view(T, H, 2, d), eps) * w["q.norm"]
     k = rms_div((h @ w["k"].T).view(T, G, 2, d), eps) * w["k.norm"]
     v = (h @ w["v"].T).view(T, G, dv)
-    lam = math.exp(float((w["lq1"] * w["lk1"]).sum())) - math.exp(float((w["lq2"] * w["lk2"]).sum())) + diff
-    vis = visible(T, int((m.get("mask") or {}).get("size") or 0))
-    heads = []
-    for a in range(H):
-        g = a // (H // G)
-        maps = [softmax_rows((q[:, a, n] @ k[:, g, n].T) * float(m["scale"]), vis) @ v[:, g] for n in range(2)]
-        heads.append(rms_div(maps[0] - lam * maps[1], eps) * (1.0 - diff))
-    return torch.cat(heads, -1) @ w["o"].T
+    lam = second_map_weight(w["lq1"], w["lk1"], w["lq2"], w["lk2"], diff)
+    o = two_map_heads(q, k, v, float(m["scale"]), lam, 1.0 - diff, int((m.get("mask") or {}).get("size") or 0), eps)
+    return o @ w["o"].T
 
 
 def feed_forward(h, w):
@@ -151,3 +170,13 @@ def forward(cfg, sd, tokens):
         after.append(x)
     y = rms_div(x, eps) * sd["final.norm"]
     return y @ sd["head"].T, torch.stack(after)
+
+
+def greedy(cfg, sd, prompt, n):
+    """The n tokens greedy decoding appends to the prompt (the whole sequence is recomputed for every token)."""
+    seq, out = list(prompt), []
+    for _ in range(n):
+        tok = int(forward(cfg, sd, seq)[0][-1].argmax())
+        out.append(tok)
+        seq.append(tok)
+    return out
