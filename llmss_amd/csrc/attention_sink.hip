@@ -312,7 +312,10 @@ void launch_sink_attn(const void* q, const void* kc, const void* vc, const void*
 // so a lane owns one slot's softmax row: cap, mask, running maximum (starting at the sink's 0) and sum need two
 // shuffles per tile. The value tile holds VCH = 16 * NVT columns of the key's value row - all groups side by side
 // when the heads' weights are mixed afterwards - and blockIdx.y also enumerates the column chunks.
-template <int DK, int NVT>
+// PRECISE: the fp32 queries and the fp32 softmax weights enter the products as the sum of two bf16 numbers (the
+// rounded value and the rounded remainder, two matrix instructions each), so scores and weighted sums are those of
+// 32-bit queries and weights; otherwise both are rounded to bf16 once.
+template <int DK, int NVT, bool PRECISE>
 __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
     const float* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
@@ -347,13 +350,18 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
   const int64_t vrow = (int64_t)GV * vdim;
   const int voff = (all ? 0 : (kvh / vshare) * vdim) + v0;
 
-  s16x8 qf[DK / 32];
+  s16x8 qf[DK / 32], ql[PRECISE ? DK / 32 : 1];
   {
     const float* qp = q + ((int64_t)(t0 + (valid ? row : 0)) * H + (valid ? h : h0)) * DK + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < DK / 32; ++ks)
 #pragma unroll
-      for (int j = 0; j < 8; ++j) qf[ks][j] = (short)f2bf(qp[32 * ks + j]);
+      for (int j = 0; j < 8; ++j) {
+        const float x = qp[32 * ks + j];
+        const bf16_t hi = f2bf(x);
+        qf[ks][j] = (short)hi;
+        if constexpr (PRECISE) ql[ks][j] = (short)f2bf(x - bf2f(hi));
+      }
   }
   f32x4 o[NVT];
 #pragma unroll
@@ -426,6 +434,7 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
       for (int ks = 0; ks < DK / 32; ++ks) {
         const s16x8 kf = *reinterpret_cast<const s16x8*>(&Ks[(kt * 16 + li) * LDK + 32 * ks + 8 * g]);
         s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], s[kt], 0, 0, 0);
+        if constexpr (PRECISE) s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, ql[ks], s[kt], 0, 0, 0);
       }
     }
     // S^T accumulators: lane (li, g) holds slot li's scores for keys kv0 + 16 kt + 4 g + i
@@ -446,18 +455,23 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float alpha = __expf(m - mx);
+    const float alpha = PRECISE ? expf(m - mx) : __expf(m - mx);
     m = mx;
     float ps = 0.f;
-    s16x8 pf[2];
+    s16x8 pf[2], pl[PRECISE ? 2 : 1];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = s[kt][i] > -1.0e29f ? __expf(s[kt][i] - mx) : 0.f;
+        const float p = s[kt][i] > -1.0e29f ? (PRECISE ? expf(s[kt][i] - mx) : __expf(s[kt][i] - mx)) : 0.f;
         const bf16_t pb = f2bf(p);
-        ps += bf2f(pb);
         pf[kt >> 1][(kt & 1) * 4 + i] = (short)pb;
+        if constexpr (PRECISE) {
+          ps += p;
+          pl[kt >> 1][(kt & 1) * 4 + i] = (short)f2bf(p - bf2f(pb));
+        } else {
+          ps += bf2f(pb);
+        }
       }
     ps += __shfl_xor(ps, 16, 64);
     ps += __shfl_xor(ps, 32, 64);
@@ -476,6 +490,7 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
         const s16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(a1));
         const s16x8 vf = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
         o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[ks], o[dt], 0, 0, 0);
+        if constexpr (PRECISE) o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl[ks], o[dt], 0, 0, 0);
       }
     }
   }
@@ -492,7 +507,8 @@ bool sink_attn_mfma_ok(int dim, int vdim) { return (dim == 32 || dim == 64 || di
 
 void launch_sink_attn_mfma(const void* q, const void* kc, const void* vc, const void* bt, int maxb, const void* cu,
                            const void* ctx, void* out, int B, int max_qlen, int H, int G, int dim, int vdim, int bs,
-                           float scale, float cap, int all, int sink, int chunk, int vshare, hipStream_t st) {
+                           float scale, float cap, int all, int sink, int chunk, int vshare, int precise,
+                           hipStream_t st) {
   if (B == 0 || max_qlen <= 0) return;
   if (G < 1 || H % G) throw std::runtime_error("sink attention: heads must be a multiple of the key/value heads");
   if (vshare < 1 || G % vshare || chunk < 0) throw std::runtime_error("sink attention: bad vshare / chunk");
@@ -511,11 +527,15 @@ void launch_sink_attn_mfma(const void* q, const void* kc, const void* vc, const 
   const int64_t gy = (int64_t)G * (rep / GE) * nvch;
   if (gy > 65535 || B > 65535) throw std::runtime_error("sink attention: too many heads or sequences");
   dim3 grid((max_qlen + rows_per_wg - 1) / rows_per_wg, (unsigned)gy, B);
-#define LAUNCH_SAM(DK_, NVT_)                                                                                       \
-  sink_attn_mfma_kernel<DK_, NVT_><<<grid, 256, 0, st>>>((const float*)q, (const bf16_t*)kc, (const bf16_t*)vc,      \
-                                                         (const int*)bt, maxb, (const int*)cu, (const int*)ctx,      \
-                                                         (float*)out, H, G, GE, vdim, bs, scale, cap, all, nvch,     \
-                                                         sink, chunk, vshare)
+#define LAUNCH_SAM1(DK_, NVT_, PR_)                                                                                 \
+  sink_attn_mfma_kernel<DK_, NVT_, PR_><<<grid, 256, 0, st>>>(                                                      \
+      (const float*)q, (const bf16_t*)kc, (const bf16_t*)vc, (const int*)bt, maxb, (const int*)cu, (const int*)ctx, \
+      (float*)out, H, G, GE, vdim, bs, scale, cap, all, nvch, sink, chunk, vshare)
+#define LAUNCH_SAM(DK_, NVT_)              \
+  do {                                     \
+    if (precise) LAUNCH_SAM1(DK_, NVT_, true); \
+    else LAUNCH_SAM1(DK_, NVT_, false);    \
+  } while (0)
   if (dim == 32) {
     if (nvt == 16) LAUNCH_SAM(32, 16);
     else if (nvt == 8) LAUNCH_SAM(32, 8);
@@ -530,6 +550,7 @@ void launch_sink_attn_mfma(const void* q, const void* kc, const void* vc, const 
     else LAUNCH_SAM(128, 4);
   }
 #undef LAUNCH_SAM
+#undef LAUNCH_SAM1
   HIP_CHECK_LAUNCH();
 }
 

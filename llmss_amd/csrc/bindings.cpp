@@ -142,7 +142,8 @@ void launch_sink_attn(const void* q, const void* kc, const void* vc, const void*
 bool sink_attn_mfma_ok(int dim, int vdim);
 void launch_sink_attn_mfma(const void* q, const void* kc, const void* vc, const void* bt, int maxb, const void* cu,
                            const void* ctx, void* out, int B, int max_qlen, int H, int G, int dim, int vdim, int bs,
-                           float scale, float cap, int all, int sink, int chunk, int vshare, hipStream_t st);
+                           float scale, float cap, int all, int sink, int chunk, int vshare, int precise,
+                           hipStream_t st);
 void launch_talk_mix(const void* O, const void* talk, float c, void* y, int64_t ldy, int T_, int H, int G, int vdim,
                      int dt, hipStream_t st);
 
@@ -417,9 +418,10 @@ PYBIND11_MODULE(_C, m) {
   m.def("sink_attn_mfma_ok", &sink_attn_mfma_ok);
   m.def("sink_attn_mfma", [](uintptr_t q, uintptr_t kc, uintptr_t vc, uintptr_t bt, int maxb, uintptr_t cu,
                              uintptr_t ctx, uintptr_t out, int B, int max_qlen, int H, int G, int dim, int vdim, int bs,
-                             float scale, float cap, int all, int sink, int chunk, int vshare, uintptr_t st) {
+                             float scale, float cap, int all, int sink, int chunk, int vshare, int precise,
+                             uintptr_t st) {
     launch_sink_attn_mfma(CP(q), CP(kc), CP(vc), CP(bt), maxb, CP(cu), CP(ctx), P(out), B, max_qlen, H, G, dim, vdim,
-                          bs, scale, cap, all, sink, chunk, vshare, S(st));
+                          bs, scale, cap, all, sink, chunk, vshare, precise, S(st));
   });
   m.def("talk_mix", [](uintptr_t O, uintptr_t talk, float c, uintptr_t y, int64_t ldy, int T, int H, int G, int vdim,
                        int dt, uintptr_t st) { launch_talk_mix(CP(O), CP(talk), c, P(y), ldy, T, H, G, vdim, dt, S(st)); });

@@ -126,7 +126,8 @@ class DiffAttention:
         # the two maps as 2 H query heads on 2 G key heads; both key heads of a pair read one value head
         O = ops.sink_attn(q, kc, vc, inp.block_tables, cu, inp.ctx_lens, 2 * H, 2 * G, spec.dim, spec.vdim, spec.scale,
                           0.0, False, max_qlen=1 if single else max(1, inp.max_seqlen),
-                          num_decode=0 if single else inp.num_decode, sink=False, chunk=spec.chunk, vshare=2)
+                          num_decode=0 if single else inp.num_decode, sink=False, chunk=spec.chunk, vshare=2,
+                          precise=True)
         y = ops.diff_combine(O, W.lam, eps, 1.0 - spec.diff, H, G, spec.vdim, dt)
         return ops.linear_f(y, W.o, dt)
 

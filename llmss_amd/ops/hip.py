@@ -957,11 +957,12 @@ def rope_angles(positions, freqs):
 
 
 LATENT_MFMA_RANKS = (64, 128, 256)  # latent ranks the MFMA extend kernel is built for (csrc/attention_extend.hip)
+_LATENT_MFMA = os.environ.get("LLMSS_LATENT_MFMA", "1") != "0"  # 0: every rank on the generic kernel (A/B runs)
 
 
 def latent_qa_dtype(cache) -> torch.dtype:
     """Storage type latent_attn wants its absorbed queries in: bf16 where the MFMA kernel runs, else fp32."""
-    if cache.is_cuda and cache.dtype == torch.bfloat16 and cache.shape[2] in LATENT_MFMA_RANKS:
+    if cache.is_cuda and cache.dtype == torch.bfloat16 and cache.shape[2] in LATENT_MFMA_RANKS and _LATENT_MFMA:
         return torch.bfloat16
     return torch.float32
 
@@ -1291,10 +1292,11 @@ _SINK_MFMA = os.environ.get("LLMSS_SINK_MFMA", "1") != "0"  # 0: every shape on 
 
 
 def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, dim, vdim, scale, softcap,
-              all_groups, max_qlen=0, num_decode=0, sink=True, chunk=0, vshare=1):
+              all_groups, max_qlen=0, num_decode=0, sink=True, chunk=0, vshare=1, precise=False):
     """``max_qlen`` (the longest portion of the step, known on the host) > 0: a bf16 cache of a shape the matrix-core
     kernel is built for runs on it, the ``num_decode`` leading single-row sequences in one launch and the portions
-    in another; everything else runs the vector kernel."""
+    in another; everything else runs the vector kernel. ``precise``: the matrix-core kernel takes queries and softmax
+    weights as two bf16 numbers each (value and remainder), for designs that define scores and weights in 32-bit."""
     T = q.shape[0]
     _rows(q, "q", heads * dim, torch.float32)
     _check(q.is_contiguous(), "q contiguous")
@@ -1324,7 +1326,8 @@ def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads, kv_heads, 
             if n > 0:
                 lib().sink_attn_mfma(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                      block_tables.data_ptr() + 4 * first * maxb, maxb, cu.data_ptr() + 4 * first,
-                                     ctx_lens.data_ptr() + 4 * first, out.data_ptr(), n, ql, *common, _stream())
+                                     ctx_lens.data_ptr() + 4 * first, out.data_ptr(), n, ql, *common,
+                                     int(bool(precise)), _stream())
     else:
         lib().sink_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), block_tables.data_ptr(),
                         block_tables.shape[1], cu.data_ptr(), ctx_lens.data_ptr(), out.data_ptr(), T, B, *common,

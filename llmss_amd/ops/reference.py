@@ -806,14 +806,15 @@ def rope_bias_cache(proj, off_q: int, off_k: int, off_v: int, bias, positions, t
 
 def sink_attn(q, k_cache, v_cache, block_tables, cu, ctx_lens, heads: int, kv_heads: int, dim: int, vdim: int,
               scale: float, softcap: float, all_groups: bool, max_qlen: int = 0, num_decode: int = 0,
-              sink: bool = True, chunk: int = 0, vshare: int = 1):
+              sink: bool = True, chunk: int = 0, vshare: int = 1, precise: bool = False):
     """Causal attention of every row over its sequence's cached keys with a sink in the softmax denominator
     (p_j = exp(s_j) / (1 + sum exp(s)); ``sink`` false: the ordinary softmax) and optionally soft-capped scores.
     ``chunk`` > 0: a row at position i sees only the keys from floor(i / chunk) * chunk on. ``vshare`` > 1: that many
     neighbouring key heads read the same value head (the value cache holds kv_heads / vshare heads). Returns fp32
     [T, heads, R]: head h's weights applied to the value rows of every group side by side (``all_groups``,
     R = kv_heads / vshare * vdim) or of its own group only (R = vdim). ``max_qlen`` (longest portion) and
-    ``num_decode`` (leading single-row sequences) only steer the choice of GPU kernel."""
+    ``num_decode`` (leading single-row sequences) and ``precise`` (32-bit queries and weights on the matrix cores)
+    only steer the GPU kernels."""
     T = q.shape[0]
     bs = k_cache.shape[1]
     rep = heads // kv_heads

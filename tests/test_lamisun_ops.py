@@ -107,7 +107,7 @@ def test_bigram_embedding_carries_the_previous_token(device, dtype, V, W, bucket
 def test_output_normed_residual_and_depth_average(device, dtype, W, n, dwa):
     T, eps = 6, 1e-5
     h0 = rnd(n + 2, T, W, seed=1) * 2
-    y, w = rnd(T, W, seed=2, dtype=dtype) * 3, (1 + 0.1 * rnd(W, seed=3)).to(dtype).double()
+    y, w = (rnd(T, W, seed=2) * 3).to(dtype).double(), (1 + 0.1 * rnd(W, seed=3)).to(dtype).double()
     wd = rnd(n + 1, seed=4).float().double() if dwa else None
     hist = h0.float().to(device).contiguous()
     out = ops.resid_norm_add(hist, n, y.to(dtype).to(device), w.to(dtype).to(device), eps,
@@ -276,7 +276,7 @@ def two_map_case(device, dtype, H, G, d, dv, lens, cuts, scale, lam, chunk, bs=1
         single = nd == len(step)
         O = ops.sink_attn(q, kc, vc, pg.bt(seqs), cu, ctx, 2 * H, 2 * G, d, dv, scale, 0.0, False,
                           max_qlen=1 if single else max(n for _, _, n in step), num_decode=0 if single else nd,
-                          sink=False, chunk=chunk, vshare=2)
+                          sink=False, chunk=chunk, vshare=2, precise=True)
         y = ops.diff_combine(O, lam, eps, mult, H, G, dv, torch.float32).cpu()
         r = 0
         for s, p0, n in step:
