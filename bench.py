@@ -82,7 +82,22 @@ def main():
                     help="instead of the headline workload: prefill / decode throughput of the Babotar design beside "
                          "the Llama family at equal size (bench/babotar_compare.py), sizes by name, one GPU")
     ap.add_argument("--babotar-kinds", default="babotar,dense", help="which of the two models --babotar runs")
+    ap.add_argument("--lamisun", nargs="?", const="w1024,w2048,w4096", default="",
+                    help="instead of the headline workload: prefill / decode throughput of the Lamisun design beside "
+                         "the Llama family at equal size (bench/lamisun_compare.py), sizes by name, one GPU")
+    ap.add_argument("--lamisun-kinds", default="lamisun,dense", help="which of the two models --lamisun runs")
     args = ap.parse_args()
+
+    if args.lamisun:
+        sys.path.insert(0, os.path.join(ROOT, "bench"))
+        import lamisun_compare
+
+        res = lamisun_compare.run(args.lamisun.split(","), args.batch_per_gpu, args.prompt_len, args.gen_len,
+                                  args.timisun_rounds,
+                                  lambda m: print(f"[bench] {m}", file=sys.stderr, flush=True),
+                                  kinds=tuple(args.lamisun_kinds.split(",")))
+        print(json.dumps(res), flush=True)
+        return
 
     if args.babotar:
         sys.path.insert(0, os.path.join(ROOT, "bench"))

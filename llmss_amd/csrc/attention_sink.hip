@@ -455,7 +455,7 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float alpha = PRECISE ? expf(m - mx) : __expf(m - mx);
+    const float alpha = __expf(m - mx);
     m = mx;
     float ps = 0.f;
     s16x8 pf[2], pl[PRECISE ? 2 : 1];
@@ -463,7 +463,7 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
     for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float p = s[kt][i] > -1.0e29f ? (PRECISE ? expf(s[kt][i] - mx) : __expf(s[kt][i] - mx)) : 0.f;
+        const float p = s[kt][i] > -1.0e29f ? __expf(s[kt][i] - mx) : 0.f;
         const bf16_t pb = f2bf(p);
         pf[kt >> 1][(kt & 1) * 4 + i] = (short)pb;
         if constexpr (PRECISE) {

@@ -78,7 +78,7 @@ class LatentAttention:
         cache = caches[i if spec.kv_from is None else spec.kv_from][0]
         qa = ops.head_absorb(qc, W.uk_t, ops.latent_qa_dtype(cache), extra=rot)
         if W.own_kv:
-            cs = model.angles(inp, W.freqs) if rot else None
+            cs = model.angles(inp, W.rot_key, W.freqs) if rot else None
             ops.latent_norm_cache(qc, H * (dim + rot), R, W.kv_norm, model.cfg.norm_eps, cache, inp.slots, rot, cs,
                                   qa if rot else None, 0, dim)
         nd = inp.num_decode if inp.kind == "extend" else 0
@@ -427,19 +427,12 @@ class LayeredLM:
             self.tap(len(w.layers) - 1, x.sum(0))
         return h
 
-    def angles(self, inp: StepInput, freqs: torch.Tensor) -> torch.Tensor:
-        """(cos, sin) [T, len(freqs), 2] of the step's positions, formed once per step and distinct rotation."""
-        key = freqs.data_ptr()
-        got = self._angles.get(key)
-        if got is None:
-            for f, cs in self._angles.values():  # another layer's table with the same steps
-                if f.shape == freqs.shape and torch.equal(f, freqs):
-                    got = (freqs, cs)
-                    break
-            if got is None:
-                got = (freqs, ops.rope_angles(inp.positions, freqs))
-            self._angles[key] = got
-        return got[1]
+    def angles(self, inp: StepInput, key: tuple, freqs: torch.Tensor) -> torch.Tensor:
+        """(cos, sin) [T, len(freqs), 2] of the step's positions, formed once per step and distinct rotation ``key``."""
+        cs = self._angles.get(key)
+        if cs is None:
+            cs = self._angles[key] = ops.rope_angles(inp.positions, freqs)
+        return cs
 
     def _postnorm_blocks(self, inp: StepInput, kv_caches) -> torch.Tensor:
         """Blocks normed on the sublayers' outputs, with input convolutions and the depth average. ``hist`` [L + 2,

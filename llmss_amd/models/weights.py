@@ -554,6 +554,7 @@ class LatentAttnWeights:
     # row of the output gate's projection inside ``qc`` (None: no gate). Rows of ``qc`` are padded to a multiple of 8.
     freqs: Optional[torch.Tensor] = None
     gate_col: Optional[int] = None
+    rot_key: Optional[tuple] = None  # (dims, base): layers with the same rotation share a step's angles
 
     def tensors(self):
         return [t for t in (self.qc, self.kv_norm, self.uk_t, self.uv, self.o, self.freqs) if t is not None]
@@ -1089,7 +1090,8 @@ def _lamisun_finish(cfg: ModelConfig, get, device, dtype) -> ModelWeights:
             mix = LatentAttnWeights(
                 qc=dev(qc), own_kv=True, kv_norm=dev(g(p + "mix.dkv.norm")),
                 uk_t=dev(_heads_t(g(p + "mix.uk"), m.heads, m.dim, m.kv_rank, i)), uv=dev(g(p + "mix.uv")),
-                o=dev(g(p + "mix.o")), freqs=freqs, gate_col=cols.get("g"))
+                o=dev(g(p + "mix.o")), freqs=freqs, gate_col=cols.get("g"),
+                rot_key=(m.rot.dims, m.rot.base) if m.rot_dim else None)
         else:
             proj, cols = _cat_rows([("q", g(p + "mix.q")), ("k", g(p + "mix.k")), ("v", g(p + "mix.v"))])
             lq1, lk1, lq2, lk2 = (g(p + "mix." + n).float() for n in ("lq1", "lk1", "lq2", "lk2"))
