@@ -19,18 +19,20 @@
 #include "anytype.h"
 
 // c = rms_norm(src[t, off : off + R]) * w, written to cache[slot[t], :R] (slot < 0: not cached) in fp32 math.
-// rot > 0: the cached row is [c | k_rot], k_rot = src[t, off + R : off + R + rot] with neighbouring pairs (2i, 2i + 1)
-// turned by cs[t, i] = (cos, sin); and every query head's rotated part - head h holds qdim plain numbers, then rot -
-// is turned the same way into qa[t, h, R : R + rot] (qa [T, H, R + rot] in its own type TQ).
+// rot > 0: the cached row is [c | k_rot], k_rot = src[t, off + R : off + R + rot] with the neighbouring pairs
+// (2i, 2i + 1), i < rdims / 2, turned by cs[t, i] = (cos, sin) and the numbers from rdims on passed unchanged; and
+// every query head's rotated part - head h holds qdim plain numbers, then rot - is turned the same way into
+// qa[t, h, R : R + rot] (qa [T, H, R + rot] in its own type TQ).
 template <typename T, typename TQ>
 __global__ __launch_bounds__(64) void latent_norm_cache_kernel(const T* __restrict__ src, int64_t lds_, int off,
                                                                const T* __restrict__ w, float eps,
                                                                T* __restrict__ cache, const int64_t* __restrict__ slots,
-                                                               int R, int rot, const float* __restrict__ cs,
-                                                               TQ* __restrict__ qa, int off_q, int H, int qdim) {
+                                                               int R, int rot, int rdims,
+                                                               const float* __restrict__ cs, TQ* __restrict__ qa,
+                                                               int off_q, int H, int qdim) {
   const int t = blockIdx.x, lane = threadIdx.x;
   const int64_t slot = slots[t];
-  const int half = rot >> 1;
+  const int half = rdims >> 1, rest = rot - rdims;
   const float* tab = cs + (int64_t)t * half * 2;
   if (rot) {
     const T* q = src + (int64_t)t * lds_ + off_q;
@@ -41,6 +43,10 @@ __global__ __launch_bounds__(64) void latent_norm_cache_kernel(const T* __restri
       const float u = El<T>::ld(p), v = El<T>::ld(p + 1), c = tab[2 * i], sn = tab[2 * i + 1];
       El<TQ>::st(dst + (int64_t)h * (R + rot) + 2 * i, u * c - v * sn);
       El<TQ>::st(dst + (int64_t)h * (R + rot) + 2 * i + 1, v * c + u * sn);
+    }
+    for (int e = lane; e < H * rest; e += 64) {
+      const int h = e / rest, i = rdims + e - h * rest;
+      El<TQ>::st(dst + (int64_t)h * (R + rot) + i, El<T>::ld(q + (int64_t)h * (qdim + rot) + qdim + i));
     }
   }
   if (slot < 0) return;
@@ -59,17 +65,19 @@ __global__ __launch_bounds__(64) void latent_norm_cache_kernel(const T* __restri
     El<T>::st(dst + R + 2 * i, u * c - v * sn);
     El<T>::st(dst + R + 2 * i + 1, v * c + u * sn);
   }
+  for (int i = rdims + lane; i < rot; i += 64) El<T>::st(dst + R + i, El<T>::ld(s + R + i));
 }
 
 // dq: storage type of qa (0 bf16, 1 fp32); only read when rot > 0
 void launch_latent_norm_cache(const void* src, int64_t ld, int off, const void* w, float eps, void* cache,
-                              const void* slots, int T_, int R, int rot, const void* cs, void* qa, int off_q, int H,
-                              int qdim, int dt, int dq, hipStream_t st) {
+                              const void* slots, int T_, int R, int rot, int rdims, const void* cs, void* qa,
+                              int off_q, int H, int qdim, int dt, int dq, hipStream_t st) {
   if (T_ == 0) return;
-  if (rot < 0 || (rot & 1)) throw std::runtime_error("latent_norm_cache: the rotated part must be even");
+  if (rot < 0 || rdims < 0 || rdims > rot || (rdims & 1))
+    throw std::runtime_error("latent_norm_cache: rotated dimensions must be even and fit the rotated part");
   DISPATCH_T(dt, T, DISPATCH_T(rot ? dq : 1, TQ, (latent_norm_cache_kernel<T, TQ><<<T_, 64, 0, st>>>(
-      (const T*)src, ld, off, (const T*)w, eps, (T*)cache, (const int64_t*)slots, R, rot, (const float*)cs, (TQ*)qa,
-      off_q, H, qdim))));
+      (const T*)src, ld, off, (const T*)w, eps, (T*)cache, (const int64_t*)slots, R, rot, rdims, (const float*)cs,
+      (TQ*)qa, off_q, H, qdim))));
   HIP_CHECK_LAUNCH();
 }
 

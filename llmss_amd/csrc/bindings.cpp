@@ -91,8 +91,8 @@ void launch_moe_gate_up_tile(const void* h, int64_t ldh, const void* wg, const v
 void launch_moe_down_tile(const void* act, const void* wd, const void* meta, void* y, int E, int maxt, int N, int F,
                           int tile_rows, hipStream_t st);
 void launch_latent_norm_cache(const void* src, int64_t ld, int off, const void* w, float eps, void* cache,
-                              const void* slots, int T_, int R, int rot, const void* cs, void* qa, int off_q, int H,
-                              int qdim, int dt, int dq, hipStream_t st);
+                              const void* slots, int T_, int R, int rot, int rdims, const void* cs, void* qa,
+                              int off_q, int H, int qdim, int dt, int dq, hipStream_t st);
 void launch_rope_angles(const void* positions, const void* freqs, void* cs, int T_, int half, hipStream_t st);
 void launch_latent_attn(const void* qa, int64_t ldq, const void* cache, const void* bt, int maxb, const void* cu_q,
                         const void* ctx_lens, void* out, int64_t ldo, int T_, int B, int H, int R, int bs, int window,
@@ -328,10 +328,10 @@ PYBIND11_MODULE(_C, m) {
     launch_moe_down_tile(CP(act), CP(wd), CP(meta), P(y), E, maxt, N, F, tile_rows, S(st));
   });
   m.def("latent_norm_cache", [](uintptr_t src, int64_t ld, int off, uintptr_t w, float eps, uintptr_t cache,
-                                uintptr_t slots, int T, int R, int rot, uintptr_t cs, uintptr_t qa, int off_q, int H,
-                                int qdim, int dt, int dq, uintptr_t st) {
-    launch_latent_norm_cache(CP(src), ld, off, CP(w), eps, P(cache), CP(slots), T, R, rot, CP(cs), P(qa), off_q, H,
-                             qdim, dt, dq, S(st));
+                                uintptr_t slots, int T, int R, int rot, int rdims, uintptr_t cs, uintptr_t qa,
+                                int off_q, int H, int qdim, int dt, int dq, uintptr_t st) {
+    launch_latent_norm_cache(CP(src), ld, off, CP(w), eps, P(cache), CP(slots), T, R, rot, rdims, CP(cs), P(qa), off_q,
+                             H, qdim, dt, dq, S(st));
   });
   m.def("rope_angles", [](uintptr_t pos, uintptr_t freqs, uintptr_t cs, int T, int half, uintptr_t st) {
     launch_rope_angles(CP(pos), CP(freqs), P(cs), T, half, S(st));

@@ -54,7 +54,8 @@ class MixerSpec:
     kv_from: Optional[int] = None
     # ``rot_dim`` > 0: every query head carries ``rot_dim`` more numbers after its ``dim`` and the down-projection
     # ``rot_dim`` more rows after the latent - one key part shared by all heads - both turned by ``rot`` (pairs of
-    # neighbours) and multiplied into the score beside the latent part; the rotated key part is cached with the latent
+    # neighbours, the first ``rot.dims`` <= rot_dim numbers; the rest pass unchanged) and multiplied into the score
+    # beside the latent part; the rotated key part is cached with the latent
     rot_dim: int = 0
     rot: Optional["RotarySpec"] = None
     gate: bool = False  # the concatenated heads are multiplied by sigmoid(W_g h) before the output projection
@@ -460,7 +461,7 @@ def _lamisun(cls, d: Dict[str, Any]) -> "ModelConfig":
             rot = None
             if rd:
                 rot = RotarySpec(int(m["rot"]["dims"]), float(m["rot"]["base"]), None, "neighbours")
-                if rot.dims != rd or rd % 2:
+                if rot.dims > rd or rot.dims % 2:
                     raise ValueError(f"Lamisun layer {i}: {rot.dims} rotary dimensions on a rotated part of {rd}")
             mixer = MixerSpec("latent_attention", int(m["heads"]), int(m["dim"]), int(m["vdim"]), int(m["kv_rank"]),
                               float(m["scale"]), 0, None, rd, rot, True)

@@ -933,17 +933,18 @@ def latent_norm_cache(src, off, R, w, eps, cache, slots, rot=0, cs=None, qa=None
            "latent cache [blocks, block_size, R + rot] in the model's storage type")
     _check(w.dtype == src.dtype and w.is_contiguous() and w.numel() == R, "latent norm weight")
     _check(slots.dtype == torch.int64 and slots.is_contiguous() and slots.numel() == T and slots.is_cuda, "slots")
-    H = dq = 0
+    H = dq = rdims = 0
     if rot:
-        _check(rot % 2 == 0, "the rotated part must be even")
         _f32c(cs, "angles")
-        _check(tuple(cs.shape) == (T, rot // 2, 2), "angles [T, rot / 2, 2]")
+        _check(cs.dim() == 3 and cs.shape[0] == T and cs.shape[2] == 2 and 2 * cs.shape[1] <= rot,
+               "angles [T, rotated dims / 2, 2], rotated dims <= rot")
+        rdims = 2 * cs.shape[1]
         _check(qa.is_contiguous() and qa.is_cuda and qa.dim() == 3 and qa.shape[0] == T and qa.shape[2] == R + rot,
                "qa [T, H, R + rot] contiguous")
         H, dq = qa.shape[1], _dt(qa, "qa")
         _check(off_q >= 0 and off_q + H * (qdim + rot) <= src.shape[1], "query columns outside src")
     lib().latent_norm_cache(src.data_ptr(), src.stride(0), int(off), w.data_ptr(), float(eps), cache.data_ptr(),
-                            slots.data_ptr(), T, R, rot, _ptr(cs) if rot else 0, _ptr(qa) if rot else 0, int(off_q), H,
+                            slots.data_ptr(), T, R, rot, rdims, _ptr(cs) if rot else 0, _ptr(qa) if rot else 0, int(off_q), H,
                             int(qdim), _dt(src, "src"), dq, _stream())
 
 

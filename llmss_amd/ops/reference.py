@@ -501,12 +501,14 @@ def head_expand(o: torch.Tensor, uv: torch.Tensor, out_dtype) -> torch.Tensor:
 
 
 def _turn_neighbours(x: torch.Tensor, cs: torch.Tensor) -> torch.Tensor:
-    """x [T, ..., rot] with pairs (2i, 2i + 1) turned by cs [T, rot / 2, 2] = (cos, sin)."""
-    T, rot = x.shape[0], x.shape[-1]
-    shape = [T] + [1] * (x.dim() - 2) + [rot // 2]
+    """x [T, ..., rot] with the pairs (2i, 2i + 1), i < cs.shape[1], turned by cs [T, dims / 2, 2] = (cos, sin); the
+    numbers from ``dims`` on pass unchanged."""
+    T, dims = x.shape[0], 2 * cs.shape[1]
+    shape = [T] + [1] * (x.dim() - 2) + [dims // 2]
     c, s = cs[..., 0].view(shape), cs[..., 1].view(shape)
-    u, v = x[..., 0::2], x[..., 1::2]
-    return torch.stack([u * c - v * s, v * c + u * s], -1).reshape(x.shape)
+    u, v = x[..., 0:dims:2], x[..., 1:dims:2]
+    turned = torch.stack([u * c - v * s, v * c + u * s], -1).reshape(*x.shape[:-1], dims)
+    return torch.cat([turned, x[..., dims:]], -1)
 
 
 def latent_norm_cache(src: torch.Tensor, off: int, R: int, w: torch.Tensor, eps: float, cache: torch.Tensor,
@@ -514,7 +516,7 @@ def latent_norm_cache(src: torch.Tensor, off: int, R: int, w: torch.Tensor, eps:
                       qa: Optional[torch.Tensor] = None, off_q: int = 0, qdim: int = 0) -> None:
     """cache[slot[t], :R] = rms_norm(src[t, off : off + R]) * w (slots < 0 are skipped); cache is [blocks, bs,
     R + rot]. ``rot`` > 0: the ``rot`` columns after the latent's are one key part shared by all heads; turned by
-    ``cs`` [T, rot / 2, 2] (neighbouring pairs) they fill the cached row, and every query head's last ``rot`` numbers
+    ``cs`` [T, dims / 2, 2] (neighbouring pairs of the first ``dims`` <= rot numbers) they fill the cached row, and every query head's last ``rot`` numbers
     (head h at src[t, off_q + h * (qdim + rot) + qdim]), turned the same way, fill qa[t, h, R:]."""
     c = src[:, off:off + R].float()
     c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * w.float()

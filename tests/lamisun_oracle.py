@@ -80,14 +80,16 @@ def softmax_rows(s, vis):
     return e / e.sum(-1, keepdim=True)
 
 
-def latent_heads(q, down, norm_w, uk, uv, H, d, r, dv, R, base, scale, eps):
-    """q [T, H * (d + r)] (per head: d plain numbers, then r that turn with the position), down [T, R + r] (the
-    latent before its norm, then one turning key part for all heads). Returns the heads' outputs [T, H * dv]."""
+def latent_heads(q, down, norm_w, uk, uv, H, d, r, dv, R, base, scale, eps, dims=None):
+    """q [T, H * (d + r)] (per head: d plain numbers, then r of which the first ``dims`` turn with the position),
+    down [T, R + r] (the latent before its norm, then one such key part for all heads). Returns the heads' outputs
+    [T, H * dv]."""
     T = q.shape[0]
+    dims = r if dims is None else dims
     q = q.view(T, H, d + r)
-    q_plain, q_rot = q[..., :d], rotate_pairs(q[..., d:], base, r)
+    q_plain, q_rot = q[..., :d], rotate_pairs(q[..., d:], base, dims)
     c = rms_div(down[:, :R], eps) * norm_w
-    k_rot = rotate_pairs(down[:, R:], base, r)
+    k_rot = rotate_pairs(down[:, R:], base, dims)
     k_plain = (c @ uk.T).view(T, H, d)
     v = (c @ uv.T).view(T, H, dv)
     vis = visible(T)
@@ -101,9 +103,8 @@ def latent_heads(q, down, norm_w, uk, uv, H, d, r, dv, R, base, scale, eps):
 def latent_attention(h, m, w, eps):
     """h [T, W]; m the mixer's config; w maps short names (q, dkv, dkv.norm, uk, uv, g, o) to tensors."""
     H, d, r, dv, R = int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"]), int(m["kv_rank"])
-    assert int(m["rot"]["dims"]) == r
     o = latent_heads(h @ w["q"].T, h @ w["dkv"].T, w["dkv.norm"], w["uk"], w["uv"], H, d, r, dv, R,
-                     float(m["rot"]["base"]), float(m["scale"]), eps)
+                     float(m["rot"]["base"]), float(m["scale"]), eps, int(m["rot"]["dims"]))
     return (o * torch.sigmoid(h @ w["g"].T)) @ w["o"].T
 
 

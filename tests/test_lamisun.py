@@ -21,10 +21,10 @@ RUNS = [pytest.param("cpu", "float32", id="cpu-fp32"), pytest.param("cuda", "flo
         pytest.param("cuda", "bfloat16", marks=gpu, id="gpu-bf16")]
 
 
-def lat(heads, dim, rot, vdim, rank, scale, base=10000.0, ff=None):
+def lat(heads, dim, rot, vdim, rank, scale, base=10000.0, ff=None, dims=None):
     return dict(type="latent_attention",
                 mixer=dict(heads=heads, dim=dim, rot_dim=rot, vdim=vdim, kv_rank=rank, scale=scale,
-                           rot=dict(base=base, dims=rot)),
+                           rot=dict(base=base, dims=rot if dims is None else dims)),
                 mlp=dict(kind="dense", ff=ff) if ff else None)
 
 
@@ -68,7 +68,7 @@ CONFIGS = {
     "odd": model(51, 36, 1e-5, 2, 1.3, 7, 5, 3, [
         att(6, 3, 6, 5, 0.4, 0.35, 5, ff=27),
         lat(5, 6, 2, 7, 10, 0.4, base=20.0, ff=19),
-        lat(3, 10, 6, 5, 14, 0.3),
+        lat(3, 10, 6, 5, 14, 0.3, dims=4),  # the last two numbers of the rotated part do not turn
     ]),
 }
 
@@ -325,7 +325,7 @@ def test_config_reader_rejects_what_the_design_does_not_have():
     with pytest.raises(ValueError):
         ModelConfig.from_hf_dict(bad)
     bad = json.loads(json.dumps(CONFIGS["mixed"]))
-    bad["layers"][0]["mixer"]["rot"]["dims"] = 2  # the rotation must cover the whole rotated part
+    bad["layers"][0]["mixer"]["rot"]["dims"] = 6  # more rotated dimensions than the rotated part holds
     with pytest.raises(ValueError):
         ModelConfig.from_hf_dict(bad)
     bad = json.loads(json.dumps(CONFIGS["plain"]))
