@@ -52,11 +52,12 @@ __global__ __launch_bounds__(256) void attn_extend_kernel(
 
   const int G = nh / nkv;
   const int rows_per_wg = 64 / GE;
-  const int b = blockIdx.z;
-  const int kvh = blockIdx.y / (G / GE);
-  const int h0 = kvh * G + (blockIdx.y % (G / GE)) * GE;  // first query head of this workgroup
+  int bx = blockIdx.x, by = blockIdx.y, b = blockIdx.z;
+  if (nsplit <= 1) causal_block_order(bx, by, b);  // (with a key split x counts the splits of one row)
+  const int kvh = by / (G / GE);
+  const int h0 = kvh * G + (by % (G / GE)) * GE;  // first query head of this workgroup
   const int t0 = cu_q[b], qlen = cu_q[b + 1] - t0;
-  const int r0 = nsplit > 1 ? 0 : blockIdx.x * rows_per_wg;
+  const int r0 = nsplit > 1 ? 0 : bx * rows_per_wg;
   if (r0 >= qlen) return;
   const int ctx = ctx_lens[b];
   const int p0 = ctx - qlen;  // position of the chunk's first token

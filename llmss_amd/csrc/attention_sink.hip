@@ -303,19 +303,25 @@ void launch_sink_attn(const void* q, const void* kc, const void* vc, const void*
   HIP_CHECK_LAUNCH();
 }
 
-// The same attention on the matrix cores, for portions of bf16 prompts (key size 64 or 128, value size a multiple
-// of 8). One workgroup serves one key/value group, GE of its query heads and 64 / GE query rows of one sequence:
-// the 64 "slots" of its four waves enumerate (row, head) pairs, slot s -> row s / GE, head s % GE, so a key tile is
-// staged in LDS once for the whole head group. Per wave (16 slots) the products are the swapped ones,
+// The same attention on the matrix cores, for portions of bf16 prompts (key size 32, 64 or 128, value size a
+// multiple of 8). One workgroup serves one key/value group, GE of its query heads and 64 * NS / GE query rows of one
+// sequence: its 64 * NS "slots" enumerate (row, head) pairs, slot s -> row s / GE, head s % GE, so a key tile is
+// staged in LDS once for the whole head group. A wave owns NS groups of 16 neighbouring slots; per group the
+// products are the swapped ones,
 //   S^T[key][slot] = K . Q^T   (A = K rows from LDS, B = Q^T fragments in registers)
 //   O^T[c][slot]  += V^T . P^T (A = V^T by transposing LDS reads, B = P^T straight from the S^T accumulators)
 // so a lane owns one slot's softmax row: cap, mask, running maximum (starting at the sink's 0) and sum need two
-// shuffles per tile. The value tile holds VCH = 16 * NVT columns of the key's value row - all groups side by side
-// when the heads' weights are mixed afterwards - and blockIdx.y also enumerates the column chunks.
+// shuffles per tile, and a key or value fragment read from LDS feeds the matrix instructions of all NS groups.
+// The softmax runs on base-2 exponents (scores times log2 e). A tile that every row of a group sees whole - before
+// the group's first position, not before the chunk of its last - skips the mask. Row blocks are taken last first and
+// spread evenly over the dies (causal_block_order). (Two tiles in LDS, the next one written while this one is read
+// and one barrier per tile, measured the same as one tile and two barriers, and is not kept.)
+// The value tile holds VCH = 16 * NVT columns of the key's value row - all groups side by side when the heads'
+// weights are mixed afterwards - and blockIdx.y also enumerates the column chunks.
 // PRECISE: the fp32 queries and the fp32 softmax weights enter the products as the sum of two bf16 numbers (the
 // rounded value and the rounded remainder, two matrix instructions each), so scores and weighted sums are those of
 // 32-bit queries and weights; otherwise both are rounded to bf16 once.
-template <int DK, int NVT, bool PRECISE>
+template <int DK, int NVT, bool PRECISE, int NS>
 __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
     const float* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q, const int* __restrict__ ctx_lens,
@@ -328,53 +334,69 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
   __shared__ __attribute__((aligned(16))) bf16_t Ks[BKV * LDK];
   __shared__ __attribute__((aligned(16))) bf16_t Vs[BKV * LDV];
   const int rep = H / G;
-  const int rows_per_wg = 64 / GE;
-  const int b = blockIdx.z;
-  const int vch = blockIdx.y % nvch, hy = blockIdx.y / nvch;
+  const int rows_per_wg = 64 * NS / GE;
+  int bx, by, b;
+  causal_block_order(bx, by, b);
+  const int vch = by % nvch, hy = by / nvch;
   const int kvh = hy / (rep / GE);
   const int h0 = kvh * rep + (hy % (rep / GE)) * GE;
   const int t0 = cu_q[b], qlen = cu_q[b + 1] - t0;
-  const int r0 = blockIdx.x * rows_per_wg;
+  const int r0 = bx * rows_per_wg;
   if (r0 >= qlen) return;
   const int p0 = ctx_lens[b] - qlen;
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
   const int li = lane & 15, g = lane >> 4;
-  const int slot = w * 16 + li;
-  const int row = r0 + slot / GE, h = h0 + slot % GE;
-  const bool valid = slot < rows_per_wg * GE && row < qlen;
-  const int qpos = p0 + (valid ? row : 0);
-  const int qlo = chunk > 0 ? (qpos / chunk) * chunk : 0;  // the first key this row sees
   const int GV = G / vshare;
   const int RVtot = all ? GV * vdim : vdim;
   const int v0 = vch * VCH;
   const int64_t vrow = (int64_t)GV * vdim;
   const int voff = (all ? 0 : (kvh / vshare) * vdim) + v0;
 
-  s16x8 qf[DK / 32], ql[PRECISE ? DK / 32 : 1];
-  {
-    const float* qp = q + ((int64_t)(t0 + (valid ? row : 0)) * H + (valid ? h : h0)) * DK + 8 * g;
+  // per slot group: the lane's slot, and (the same in every lane) the positions the group's rows span
+  int row[NS], hd[NS], qpos[NS], qlo[NS];
+  bool valid[NS], grp_rows[NS];
+  int grp_first[NS], grp_last[NS], grp_lo[NS], grp_hilo[NS];
+  s16x8 qf[NS][DK / 32], ql[NS][PRECISE ? DK / 32 : 1];
+  f32x4 o[NS][NVT];
+  float m[NS], lsum[NS];
+  bool wave_rows = false;
+#pragma unroll
+  for (int n = 0; n < NS; ++n) {
+    const int gs = (w * NS + n) * 16, slot = gs + li;
+    row[n] = r0 + slot / GE;
+    hd[n] = h0 + slot % GE;
+    valid[n] = slot < rows_per_wg * GE && row[n] < qlen;
+    qpos[n] = p0 + (valid[n] ? row[n] : 0);
+    qlo[n] = chunk > 0 ? (qpos[n] / chunk) * chunk : 0;  // the first key this row sees
+    // a group none of whose slots holds a row (a single decoded row fills part of the first) only helps to stage
+    grp_rows[n] = r0 + gs / GE < qlen && gs < rows_per_wg * GE;
+    wave_rows = wave_rows || grp_rows[n];
+    grp_first[n] = p0 + min(qlen - 1, r0 + gs / GE);
+    grp_last[n] = p0 + min(qlen - 1, r0 + (gs + 15) / GE);
+    grp_lo[n] = chunk > 0 ? (grp_first[n] / chunk) * chunk : 0;
+    grp_hilo[n] = chunk > 0 ? (grp_last[n] / chunk) * chunk : 0;
+    const float* qp = q + ((int64_t)(t0 + (valid[n] ? row[n] : 0)) * H + (valid[n] ? hd[n] : h0)) * DK + 8 * g;
 #pragma unroll
     for (int ks = 0; ks < DK / 32; ++ks)
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const float x = qp[32 * ks + j];
         const bf16_t hi = f2bf(x);
-        qf[ks][j] = (short)hi;
-        if constexpr (PRECISE) ql[ks][j] = (short)f2bf(x - bf2f(hi));
+        qf[n][ks][j] = (short)hi;
+        if constexpr (PRECISE) ql[n][ks][j] = (short)f2bf(x - bf2f(hi));
       }
-  }
-  f32x4 o[NVT];
 #pragma unroll
-  for (int i = 0; i < NVT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  // the sink: score 0, weight exp(0 - m), no value; without it a masked score's stand-in is the starting maximum
-  float m = sink ? 0.f : -1.0e30f, lsum = sink ? 1.f : 0.f;
+    for (int i = 0; i < NVT; ++i) o[n][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // the sink: score 0, weight exp(0 - m), no value; without it a masked score's stand-in is the starting maximum
+    m[n] = sink ? 0.f : -1.0e30f;
+    lsum[n] = sink ? 1.f : 0.f;
+  }
+  constexpr float kLog2e = 1.4426950408889634f;
   const float icap = cap > 0.f ? 1.0f / cap : 0.f;
+  const float scale2 = scale * kLog2e;
   const int r_last = min(qlen, r0 + rows_per_wg) - 1;
   const int kv_end = p0 + r_last + 1;
   const int kv_begin = chunk > 0 ? ((p0 + r0) / chunk) * chunk : 0;  // the first row's block starts first
-  const int wave_qhi = p0 + min(qlen - 1, r0 + (16 * w + 15) / GE);
-  const int wave_first = p0 + min(qlen - 1, r0 + (16 * w) / GE);
-  const int wave_lo = chunk > 0 ? (wave_first / chunk) * chunk : 0;
   const int* bt = block_tables + (int64_t)b * max_blocks;
   constexpr int CHK = DK / 8, CHV = VCH / 8;
   // Software pipeline: the next tile's 16-byte chunks are fetched into registers while this tile is computed from
@@ -414,71 +436,98 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
       *reinterpret_cast<u16x8*>(&Vs[(c / CHV) * LDV + (c % CHV) * 8]) = vr[j];
     }
   };
-  // a wave none of whose slots holds a row (a single decoded row fills part of the first wave) only helps to stage
-  const bool wave_rows = r0 + (16 * w) / GE < qlen && 16 * w < rows_per_wg * GE;
-  if (kv_end > kv_begin) load_tile(kv_begin);  // (a padded row has no keys at all)
-  for (int kv0 = kv_begin; kv0 < kv_end; kv0 += BKV) {
-    __syncthreads();  // every wave is done reading the previous tile
-    store_tile();
-    __syncthreads();
-    if (kv0 + BKV < kv_end) load_tile(kv0 + BKV);
-    if (!wave_rows) continue;
-    if (kv0 > wave_qhi) continue;  // whole tile in this wave's causal future (barriers stay uniform)
-    if (kv0 + BKV <= wave_lo) continue;  // whole tile before the block of this wave's first row
-
-    f32x4 s[4];
+  // one tile of keys from LDS for every slot group of this wave that sees any of it
+  auto compute_tile = [&](int kv0) {
+    bool act[NS];
+    bool any = false;
+#pragma unroll
+    for (int n = 0; n < NS; ++n) {
+      // not wholly in the group's causal future, not wholly before the block of its first row
+      act[n] = grp_rows[n] && kv0 <= grp_last[n] && kv0 + BKV > grp_lo[n];
+      any = any || act[n];
+    }
+    if (!any) return;
+    f32x4 s[NS][4];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
-      s[kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int n = 0; n < NS; ++n) s[n][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < DK / 32; ++ks) {
         const s16x8 kf = *reinterpret_cast<const s16x8*>(&Ks[(kt * 16 + li) * LDK + 32 * ks + 8 * g]);
-        s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[ks], s[kt], 0, 0, 0);
-        if constexpr (PRECISE) s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, ql[ks], s[kt], 0, 0, 0);
+#pragma unroll
+        for (int n = 0; n < NS; ++n) {
+          s[n][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[n][ks], s[n][kt], 0, 0, 0);
+          if constexpr (PRECISE) s[n][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, ql[n][ks], s[n][kt], 0, 0, 0);
+        }
       }
     }
-    // S^T accumulators: lane (li, g) holds slot li's scores for keys kv0 + 16 kt + 4 g + i
-    float mx = m;
+    // S^T accumulators: lane (li, g) holds slot li's scores for keys kv0 + 16 kt + 4 g + i.
+    // The matrix instructions above and below run for every group of the wave (a fragment from LDS serves them all);
+    // a group that sees nothing of the tile gets zero weights, which leave its sums as they are.
+    s16x8 pf[NS][2], pl[NS][PRECISE ? 2 : 1];
+    auto softmax = [&](int n, auto whole_c, auto cap_c) {
+      constexpr bool WHOLE = decltype(whole_c)::value, CAP = decltype(cap_c)::value;
+      float mx = m[n];
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt)
+      for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = kv0 + kt * 16 + 4 * g + i;
-        float v = s[kt][i] * scale;
-        if (cap > 0.f) {
-          const float e2 = __expf(2.0f * v * icap);  // tanh(x) = 1 - 2 / (exp(2x) + 1)
-          v = cap * (1.0f - 2.0f / (e2 + 1.0f));
+        for (int i = 0; i < 4; ++i) {
+          float v;
+          if constexpr (CAP) {
+            const float x = s[n][kt][i] * scale;
+            const float e2 = __expf(2.0f * x * icap);  // tanh(x) = 1 - 2 / (exp(2x) + 1)
+            v = cap * (1.0f - 2.0f / (e2 + 1.0f)) * kLog2e;
+          } else {
+            v = s[n][kt][i] * scale2;
+          }
+          if constexpr (!WHOLE) {
+            const int key = kv0 + kt * 16 + 4 * g + i;
+            v = (key <= qpos[n] && key >= qlo[n] && key < kv_end) ? v : -1.0e30f;
+          }
+          s[n][kt][i] = v;
+          mx = fmaxf(mx, v);
         }
-        v = (key <= qpos && key >= qlo && key < kv_end) ? v : -1.0e30f;
-        s[kt][i] = v;
-        mx = fmaxf(mx, v);
-      }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float alpha = __expf(m - mx);
-    m = mx;
-    float ps = 0.f;
-    s16x8 pf[2], pl[PRECISE ? 2 : 1];
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float alpha = __builtin_amdgcn_exp2f(m[n] - mx);
+      m[n] = mx;
+      float ps = 0.f;
 #pragma unroll
-    for (int kt = 0; kt < 4; ++kt)
+      for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float p = s[kt][i] > -1.0e29f ? __expf(s[kt][i] - mx) : 0.f;
-        const bf16_t pb = f2bf(p);
-        pf[kt >> 1][(kt & 1) * 4 + i] = (short)pb;
-        if constexpr (PRECISE) {
-          ps += p;
-          pl[kt >> 1][(kt & 1) * 4 + i] = (short)f2bf(p - bf2f(pb));
-        } else {
-          ps += bf2f(pb);
+        for (int i = 0; i < 4; ++i) {
+          float p = __builtin_amdgcn_exp2f(s[n][kt][i] - mx);
+          if constexpr (!WHOLE) p = s[n][kt][i] > -1.0e29f ? p : 0.f;
+          const bf16_t pb = f2bf(p);
+          pf[n][kt >> 1][(kt & 1) * 4 + i] = (short)pb;
+          if constexpr (PRECISE) {
+            ps += p;
+            pl[n][kt >> 1][(kt & 1) * 4 + i] = (short)f2bf(p - bf2f(pb));
+          } else {
+            ps += bf2f(pb);
+          }
         }
-      }
-    ps += __shfl_xor(ps, 16, 64);
-    ps += __shfl_xor(ps, 32, 64);
-    lsum = lsum * alpha + ps;
+      ps += __shfl_xor(ps, 16, 64);
+      ps += __shfl_xor(ps, 32, 64);
+      lsum[n] = lsum[n] * alpha + ps;
 #pragma unroll
-    for (int i = 0; i < NVT; ++i) o[i] *= alpha;
-
+      for (int i = 0; i < NVT; ++i) o[n][i] *= alpha;
+    };
+#pragma unroll
+    for (int n = 0; n < NS; ++n) {
+      if (!act[n]) {
+        const s16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+        pf[n][0] = pf[n][1] = z;
+        if constexpr (PRECISE) pl[n][0] = pl[n][1] = z;
+        continue;
+      }
+      // does every row of the group see the whole tile?
+      const bool whole = kv0 + BKV - 1 <= grp_first[n] && kv0 >= grp_hilo[n];
+      if (cap > 0.f) softmax(n, std::false_type{}, std::true_type{});
+      else if (whole) softmax(n, std::true_type{}, std::false_type{});
+      else softmax(n, std::false_type{}, std::false_type{});
+    }
     const int tq = li >> 2, tp = li & 3;
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
@@ -489,17 +538,31 @@ __global__ __launch_bounds__(256, 2) void sink_attn_mfma_kernel(
         const s16x4 x0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(a0));
         const s16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(a1));
         const s16x8 vf = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
-        o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[ks], o[dt], 0, 0, 0);
-        if constexpr (PRECISE) o[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl[ks], o[dt], 0, 0, 0);
+#pragma unroll
+        for (int n = 0; n < NS; ++n) {
+          o[n][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[n][ks], o[n][dt], 0, 0, 0);
+          if constexpr (PRECISE) o[n][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl[n][ks], o[n][dt], 0, 0, 0);
+        }
       }
     }
+  };
+  if (kv_end > kv_begin) load_tile(kv_begin);  // (a padded row has no keys at all)
+  for (int kv0 = kv_begin; kv0 < kv_end; kv0 += BKV) {
+    __syncthreads();  // every wave is done reading the previous tile
+    store_tile();
+    __syncthreads();
+    if (kv0 + BKV < kv_end) load_tile(kv0 + BKV);
+    if (wave_rows) compute_tile(kv0);
   }
-  if (!valid) return;
-  const float inv = 1.0f / lsum;
-  float* op = out + ((int64_t)(t0 + row) * H + h) * RVtot + v0 + 4 * g;
 #pragma unroll
-  for (int dt = 0; dt < NVT; ++dt)
-    if (v0 + dt * 16 + 4 * g < RVtot) *reinterpret_cast<f32x4*>(op + dt * 16) = o[dt] * inv;
+  for (int n = 0; n < NS; ++n) {
+    if (!valid[n]) continue;
+    const float inv = 1.0f / lsum[n];
+    float* op = out + ((int64_t)(t0 + row[n]) * H + hd[n]) * RVtot + v0 + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < NVT; ++dt)
+      if (v0 + dt * 16 + 4 * g < RVtot) *reinterpret_cast<f32x4*>(op + dt * 16) = o[n][dt] * inv;
+  }
 }
 
 // Can the matrix-core kernel take this shape? (bf16 storage is the caller's to check.)
@@ -520,37 +583,43 @@ void launch_sink_attn_mfma(const void* q, const void* kc, const void* vc, const 
       GE = ge;
       break;
     }
-  const int rows_per_wg = 64 / GE;
   const int RVtot = all ? (G / vshare) * vdim : vdim;
   const int nvt = RVtot > 128 ? 16 : (RVtot > 64 ? 8 : 4);
   const int nvch = (RVtot + nvt * 16 - 1) / (nvt * 16);
+  // two slot groups per wave where a portion has more rows than one group each would hold (the widest value tile,
+  // and 128-wide keys with split queries beside the middle one, keep one: two groups would not fit the registers)
+  const bool two_fit = nvt <= 4 || (nvt == 8 && !(dim == 128 && precise));
+  const int ns = (two_fit && max_qlen > 64 / GE) ? 2 : 1;
+  const int rows_per_wg = 64 * ns / GE;
   const int64_t gy = (int64_t)G * (rep / GE) * nvch;
   if (gy > 65535 || B > 65535) throw std::runtime_error("sink attention: too many heads or sequences");
   dim3 grid((max_qlen + rows_per_wg - 1) / rows_per_wg, (unsigned)gy, B);
-#define LAUNCH_SAM1(DK_, NVT_, PR_)                                                                                 \
-  sink_attn_mfma_kernel<DK_, NVT_, PR_><<<grid, 256, 0, st>>>(                                                      \
+#define LAUNCH_SAM2(DK_, NVT_, PR_, NS_)                                                                            \
+  sink_attn_mfma_kernel<DK_, NVT_, PR_, NS_><<<grid, 256, 0, st>>>(                                                 \
       (const float*)q, (const bf16_t*)kc, (const bf16_t*)vc, (const int*)bt, maxb, (const int*)cu, (const int*)ctx, \
       (float*)out, H, G, GE, vdim, bs, scale, cap, all, nvch, sink, chunk, vshare)
-#define LAUNCH_SAM(DK_, NVT_)              \
-  do {                                     \
-    if (precise) LAUNCH_SAM1(DK_, NVT_, true); \
-    else LAUNCH_SAM1(DK_, NVT_, false);    \
+#define LAUNCH_SAM1(DK_, NVT_, NS_)                                                       \
+  do {                                                                                    \
+    if (!precise) LAUNCH_SAM2(DK_, NVT_, false, NS_);                                     \
+    else LAUNCH_SAM2(DK_, NVT_, true, (DK_ == 128 && NVT_ == 8 && NS_ == 2) ? 1 : NS_);   \
   } while (0)
-  if (dim == 32) {
-    if (nvt == 16) LAUNCH_SAM(32, 16);
-    else if (nvt == 8) LAUNCH_SAM(32, 8);
-    else LAUNCH_SAM(32, 4);
-  } else if (dim == 64) {
-    if (nvt == 16) LAUNCH_SAM(64, 16);
-    else if (nvt == 8) LAUNCH_SAM(64, 8);
-    else LAUNCH_SAM(64, 4);
-  } else {
-    if (nvt == 16) LAUNCH_SAM(128, 16);
-    else if (nvt == 8) LAUNCH_SAM(128, 8);
-    else LAUNCH_SAM(128, 4);
-  }
+#define LAUNCH_SAM(DK_)                       \
+  do {                                        \
+    if (nvt == 16) LAUNCH_SAM1(DK_, 16, 1);   \
+    else if (nvt == 8) {                      \
+      if (ns == 2) LAUNCH_SAM1(DK_, 8, 2);    \
+      else LAUNCH_SAM1(DK_, 8, 1);            \
+    } else {                                  \
+      if (ns == 2) LAUNCH_SAM1(DK_, 4, 2);    \
+      else LAUNCH_SAM1(DK_, 4, 1);            \
+    }                                         \
+  } while (0)
+  if (dim == 32) LAUNCH_SAM(32);
+  else if (dim == 64) LAUNCH_SAM(64);
+  else LAUNCH_SAM(128);
 #undef LAUNCH_SAM
 #undef LAUNCH_SAM1
+#undef LAUNCH_SAM2
   HIP_CHECK_LAUNCH();
 }
 

@@ -36,6 +36,19 @@ __device__ __forceinline__ bf16_t f2bf(float f) {
   return *reinterpret_cast<bf16_t*>(&h);
 }
 
+// Block order for causal attention grids (x: row blocks of a sequence, y: heads, z: sequences). A later row block
+// walks more keys, and the hardware hands out workgroups in the order x, y, z, one die after the other: taken as
+// they come, the longest workgroups start last and each die gets its own residues of x. Here the linear workgroup
+// number picks the row block from the last one down and walks (y, z) fastest, so long workgroups start first,
+// every die gets every row block equally often, and a die keeps to the same heads' keys.
+__device__ __forceinline__ void causal_block_order(int& bx, int& by, int& bz) {
+  const int id = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+  const int S = gridDim.y * gridDim.z;
+  bx = gridDim.x - 1 - id / S;
+  by = (id % S) % gridDim.y;
+  bz = (id % S) / gridDim.y;
+}
+
 __device__ __forceinline__ float warp_sum(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
