@@ -19,9 +19,10 @@ sys.path.insert(0, os.path.join(ROOT, "bench"))
 PEAK_TFLOPS, PEAK_TBS = 2500.0, 8.0
 
 
-def timed(fn, iters=10, warm=2):
+def timed(fn, iters=10, warm=2, reps=1):
     """Device seconds per call: the call is captured into a HIP graph and the graph replayed, so the host-side
-    launcher (argument checks, allocations) is not part of the time."""
+    launcher (argument checks, allocations) is not part of the time. ``reps`` > 1 captures that many calls back to
+    back, as a decode graph holds a kernel among many others: the floor of replaying a graph is then shared."""
     for _ in range(warm):
         fn()
     torch.cuda.synchronize()
@@ -33,7 +34,8 @@ def timed(fn, iters=10, warm=2):
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     with torch.cuda.graph(g):
-        fn()
+        for _ in range(reps):
+            fn()
     g.replay()
     torch.cuda.synchronize()
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -42,7 +44,7 @@ def timed(fn, iters=10, warm=2):
         g.replay()
     b.record()
     b.synchronize()
-    return a.elapsed_time(b) / iters * 1e-3
+    return a.elapsed_time(b) / (iters * reps) * 1e-3
 
 
 def main():

@@ -721,11 +721,75 @@ __global__ __launch_bounds__(256) void qk_norm_cache_kernel(const T* __restrict_
     for (int e = threadIdx.x; e < G * vdim; e += blockDim.x) vc[slot * (int64_t)G * vdim + e] = row[off_v + e];
 }
 
+// The same for bf16 rows whose vectors are whole 16-byte pieces: dim / 8 neighbouring lanes (a power of two) share a
+// vector, each lane reads its eight numbers once, the sum of squares goes round the lanes of the vector, and the
+// result leaves in 16-byte stores (two for a query's eight fp32 numbers).
+__global__ __launch_bounds__(256) void qk_norm_cache_vec_kernel(const bf16_t* __restrict__ proj, int64_t ldp,
+                                                                int off_q, int off_k, int off_v,
+                                                                const bf16_t* __restrict__ qw,
+                                                                const bf16_t* __restrict__ kw, float eps,
+                                                                float* __restrict__ qout, bf16_t* __restrict__ kc,
+                                                                bf16_t* __restrict__ vc,
+                                                                const int64_t* __restrict__ slots, int H, int G,
+                                                                int maps, int dim, int vdim) {
+  const int t = blockIdx.x;
+  const int L = dim >> 3;  // lanes per vector
+  const int sub = threadIdx.x & (L - 1), per = blockDim.x / L;
+  const bf16_t* row = proj + (int64_t)t * ldp;
+  const int64_t slot = slots[t];
+  const int rep = H / G, nqv = H * maps, nkv = G * maps;
+  for (int n = threadIdx.x / L; n < nqv + nkv; n += per) {
+    const bool isk = n >= nqv;
+    const int idx = isk ? n - nqv : n;
+    if (isk && slot < 0) continue;
+    const bf16_t* wt = isk ? kw : qw;
+    const u16x8 raw = *reinterpret_cast<const u16x8*>(row + (isk ? off_k : off_q) + (int64_t)idx * dim + 8 * sub);
+    float x[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) x[i] = bf2f(raw[i]);
+    if (wt) {
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss = fmaf(x[i], x[i], ss);
+      for (int o = L >> 1; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+      const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+      const u16x8 wr = *reinterpret_cast<const u16x8*>(wt + 8 * sub);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) x[i] = x[i] * inv * bf2f(wr[i]);
+    }
+    if (isk) {
+      u16x8 y;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) y[i] = wt ? f2bf(x[i]) : raw[i];
+      *reinterpret_cast<u16x8*>(kc + (slot * nkv + idx) * (int64_t)dim + 8 * sub) = y;
+    } else {
+      const int h = idx / maps, mp = idx - h * maps;
+      const int g = h / rep, r = h - g * rep;
+      float* dst = qout + ((int64_t)t * nqv + (g * maps + mp) * rep + r) * dim + 8 * sub;
+      *reinterpret_cast<f32x4*>(dst) = f32x4{x[0], x[1], x[2], x[3]};
+      *reinterpret_cast<f32x4*>(dst + 4) = f32x4{x[4], x[5], x[6], x[7]};
+    }
+  }
+  if (slot >= 0)
+    for (int e = threadIdx.x * 8; e < G * vdim; e += blockDim.x * 8)
+      *reinterpret_cast<u16x8*>(vc + slot * (int64_t)G * vdim + e) = *reinterpret_cast<const u16x8*>(row + off_v + e);
+}
+
 void launch_qk_norm_cache(const void* proj, int64_t ldp, int off_q, int off_k, int off_v, const void* qw,
                           const void* kw, float eps, void* qout, void* kc, void* vc, const void* slots, int T_, int H,
                           int G, int maps, int dim, int vdim, int dt, hipStream_t st) {
   if (T_ == 0) return;
   if (G < 1 || H % G || maps < 1) throw std::runtime_error("qk_norm_cache: heads must be a multiple of the key heads");
+  const auto al16 = [](const void* p) { return p == nullptr || ((uintptr_t)p & 15) == 0; };
+  if (dt == 0 && dim >= 8 && dim <= 512 && (dim & (dim - 1)) == 0 && (G * vdim) % 8 == 0 && ldp % 8 == 0 &&
+      off_q % 8 == 0 && off_k % 8 == 0 && off_v % 8 == 0 && al16(proj) && al16(qw) && al16(kw) && al16(qout) &&
+      al16(kc) && al16(vc)) {
+    qk_norm_cache_vec_kernel<<<T_, 256, 0, st>>>((const bf16_t*)proj, ldp, off_q, off_k, off_v, (const bf16_t*)qw,
+                                                 (const bf16_t*)kw, eps, (float*)qout, (bf16_t*)kc, (bf16_t*)vc,
+                                                 (const int64_t*)slots, H, G, maps, dim, vdim);
+    HIP_CHECK_LAUNCH();
+    return;
+  }
   DISPATCH_T(dt, T, (qk_norm_cache_kernel<T><<<T_, 256, 0, st>>>(
       (const T*)proj, ldp, off_q, off_k, off_v, (const T*)qw, (const T*)kw, eps, (float*)qout, (T*)kc, (T*)vc,
       (const int64_t*)slots, H, G, maps, dim, vdim)));

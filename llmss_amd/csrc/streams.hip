@@ -160,6 +160,109 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const TI* __restrict__
   }
 }
 
+// The same for steps of long portions: a workgroup takes CONV_STRIP neighbouring rows and a thread CH neighbouring
+// channels of them (four: 16-byte reads of fp32 rows), so an input is read once (plus the rows before the strip)
+// instead of once per tap. The rows are loaded up front, all loads in flight together; the strip's place in its
+// sequence is found once and walked from there (looked up again where a sequence ends). Taps are added in the order
+// of the kernel above: the same numbers bit for bit. RMAX: the most rows back that a tap may reach (taps - 1).
+#define CONV_STRIP 16
+template <typename T, int CH>
+__device__ __forceinline__ void conv_ld(const T* p, float* v) {
+  if constexpr (CH == 4 && sizeof(T) == 4) {
+    const f32x4 x = *reinterpret_cast<const f32x4*>(p);
+    v[0] = x[0], v[1] = x[1], v[2] = x[2], v[3] = x[3];
+  } else if constexpr (CH == 4) {
+    const u32x2 x = *reinterpret_cast<const u32x2*>(p);
+    v[0] = __uint_as_float(x[0] << 16), v[1] = __uint_as_float(x[0] & 0xffff0000u);
+    v[2] = __uint_as_float(x[1] << 16), v[3] = __uint_as_float(x[1] & 0xffff0000u);
+  } else {
+#pragma unroll
+    for (int e = 0; e < CH; ++e) v[e] = El<T>::ld(p + e);
+  }
+}
+template <typename T, int CH>
+__device__ __forceinline__ void conv_st(T* p, const float* v) {
+  if constexpr (CH == 4 && sizeof(T) == 4) {
+    *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]};
+  } else if constexpr (CH == 4) {
+    u32x2 x;
+    x[0] = (unsigned)f2bf(v[0]) | ((unsigned)f2bf(v[1]) << 16);
+    x[1] = (unsigned)f2bf(v[2]) | ((unsigned)f2bf(v[3]) << 16);
+    *reinterpret_cast<u32x2*>(p) = x;
+  } else {
+#pragma unroll
+    for (int e = 0; e < CH; ++e) El<T>::st(p + e, v[e]);
+  }
+}
+
+template <typename TI, typename TW, typename TO, int RMAX, int CH>
+__global__ __launch_bounds__(256) void causal_conv_strip_kernel(const TI* __restrict__ in, int64_t ldi,
+                                                                const TW* __restrict__ w,
+                                                                const float* __restrict__ state,
+                                                                const int* __restrict__ cu, const int* __restrict__ ctx,
+                                                                const int* __restrict__ sslots, TO* __restrict__ out,
+                                                                int64_t ldo, int B, int C, int taps, int res, int silu,
+                                                                int T_) {
+  const int t0 = blockIdx.x * CONV_STRIP;
+  const int c = (blockIdx.y * blockDim.x + threadIdx.x) * CH;
+  if (c >= C) return;  // (C is a multiple of CH)
+  const int R = taps - 1;
+  float wd[RMAX + 1][CH];  // wd[d]: the weight of the input d rows back
+#pragma unroll
+  for (int d = 0; d <= RMAX; ++d)
+#pragma unroll
+    for (int e = 0; e < CH; ++e) wd[d][e] = d <= R ? El<TW>::ld(w + (int64_t)(c + e) * taps + (R - d)) : 0.f;
+  float x[CONV_STRIP + RMAX][CH];  // x[i]: input row t0 - RMAX + i
+#pragma unroll
+  for (int i = 0; i < CONV_STRIP + RMAX; ++i) {
+    const int tt = t0 - RMAX + i;
+    if (i >= RMAX - R && tt >= 0 && tt < T_) {
+      conv_ld<TI, CH>(in + (int64_t)tt * ldi + c, x[i]);
+    } else {
+#pragma unroll
+      for (int e = 0; e < CH; ++e) x[i][e] = 0.f;
+    }
+  }
+  RowSeq r = row_seq(cu, ctx, B, t0);
+#pragma unroll
+  for (int i = 0; i < CONV_STRIP; ++i) {
+    const int t = t0 + i;
+    if (t >= T_) break;
+    if (i > 0) {
+      ++r.j;
+      ++r.pos;
+      if (r.j >= r.qlen) r = row_seq(cu, ctx, B, t);
+    }
+    float acc[CH];
+#pragma unroll
+    for (int e = 0; e < CH; ++e) acc[e] = 0.f;
+    if (r.pos >= 0) {
+      if (res) {
+#pragma unroll
+        for (int e = 0; e < CH; ++e) acc[e] = x[i + RMAX][e];
+      }
+#pragma unroll
+      for (int d = RMAX; d >= 0; --d) {
+        if (d > R || r.pos - d < 0) continue;
+        float v[CH];
+        if (r.j - d >= 0) {
+#pragma unroll
+          for (int e = 0; e < CH; ++e) v[e] = x[i + RMAX - d][e];
+        } else {
+          conv_ld<float, CH>(state + ((int64_t)sslots[r.b] * R + (r.j - d + R)) * C + c, v);
+        }
+#pragma unroll
+        for (int e = 0; e < CH; ++e) acc[e] = fmaf(wd[d][e], v[e], acc[e]);
+      }
+      if (silu) {
+#pragma unroll
+        for (int e = 0; e < CH; ++e) acc[e] = acc[e] / (1.0f + expf(-acc[e]));
+      }
+    }
+    conv_st<TO, CH>(out + (int64_t)t * ldo + c, acc);
+  }
+}
+
 // The tail after the step: state[slot, i, c] <- input at position ctx - (taps - 1) + i
 template <typename TI>
 __global__ __launch_bounds__(256) void conv_tail_kernel(const TI* __restrict__ in, int64_t ldi,
@@ -191,10 +294,29 @@ template <typename TI, typename TW, typename TO>
 static void causal_conv_t(const void* in, int64_t ldi, const void* w, void* state, const void* cu, const void* ctx,
                           const void* sslots, void* out, int64_t ldo, int T_, int B, int C, int taps, int res,
                           int silu, hipStream_t st) {
-  dim3 g(T_, (C + 256 * CONV_CPT - 1) / (256 * CONV_CPT));
-  causal_conv_kernel<TI, TW, TO><<<g, 256, 0, st>>>((const TI*)in, ldi, (const TW*)w, (const float*)state,
-                                                    (const int*)cu, (const int*)ctx, (const int*)sslots, (TO*)out, ldo,
-                                                    B, C, taps, res, silu);
+  if (T_ >= 256 && T_ >= 8 * B) {  // portions of eight rows and more on average
+    const auto al16 = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+    const bool four = C % 4 == 0 && ldi % 4 == 0 && ldo % 4 == 0 && al16(in) && al16(out) && al16(state);
+#define LAUNCH_STRIP(RMAX_, CH_)                                                                                    \
+  causal_conv_strip_kernel<TI, TW, TO, RMAX_, CH_><<<g, 256, 0, st>>>(                                              \
+      (const TI*)in, ldi, (const TW*)w, (const float*)state, (const int*)cu, (const int*)ctx, (const int*)sslots,   \
+      (TO*)out, ldo, B, C, taps, res, silu, T_)
+    if (four) {
+      dim3 g((T_ + CONV_STRIP - 1) / CONV_STRIP, (C / 4 + 255) / 256);
+      if (taps <= 4) LAUNCH_STRIP(3, 4);
+      else LAUNCH_STRIP(MAX_TAIL, 4);
+    } else {
+      dim3 g((T_ + CONV_STRIP - 1) / CONV_STRIP, (C + 255) / 256);
+      if (taps <= 4) LAUNCH_STRIP(3, 1);
+      else LAUNCH_STRIP(MAX_TAIL, 1);
+    }
+#undef LAUNCH_STRIP
+  } else {
+    dim3 g(T_, (C + 256 * CONV_CPT - 1) / (256 * CONV_CPT));
+    causal_conv_kernel<TI, TW, TO><<<g, 256, 0, st>>>((const TI*)in, ldi, (const TW*)w, (const float*)state,
+                                                      (const int*)cu, (const int*)ctx, (const int*)sslots, (TO*)out,
+                                                      ldo, B, C, taps, res, silu);
+  }
   if (taps > 1) {
     dim3 g2(B, (C + 255) / 256);
     conv_tail_kernel<TI><<<g2, 256, 0, st>>>((const TI*)in, ldi, (float*)state, (const int*)cu, (const int*)ctx,

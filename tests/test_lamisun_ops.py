@@ -154,6 +154,33 @@ def test_input_convolution_reads_the_fp32_residual(device, dtype, taps):
     close(got, x.float().double() + oracle.causal_conv(x.float().double(), w), torch.float32, "x + conv(x)")
 
 
+@pytest.mark.parametrize("device,dtype", RUNS)
+@pytest.mark.parametrize("taps", [1, 2, 4, 9])
+@pytest.mark.parametrize("C", [300, 21])
+def test_input_convolution_over_long_portions(device, dtype, taps, C):
+    """Steps of several hundred rows (on a GPU the kernel that walks strips of rows): sequences of unequal length
+    side by side, sequence ends inside a strip and at its first row, an empty portion's neighbour, portions that
+    continue from the tail, and widths that are no multiple of the workgroup or of a 16-byte read."""
+    lens = [333, 17, 290, 64]
+    cuts = [[16, 317], [16, 1], [290], [48, 16]]  # 370 rows of four sequences, then 334 rows of three
+    xs = [rnd(n, C, seed=10 + i) for i, n in enumerate(lens)]
+    w = rnd(C, taps, seed=2, dtype=dtype)
+    state = torch.full((4, max(taps - 1, 1), C), -3.0, device=device)[:, :taps - 1].contiguous()
+    got = [torch.zeros(n, C) for n in lens]
+    for step in steps_of(cuts):
+        cu, ctx, ss = meta(step, [2, 0, 3, 1], device)
+        x = torch.cat([xs[s][p0:p0 + k] for s, p0, k in step]).float().to(device)
+        y = ops.causal_conv(x, w.to(dtype).to(device), state if taps > 1 else None, cu, ctx, ss, True, False,
+                            torch.float32).cpu()
+        at = 0
+        for s, p0, k in step:
+            got[s][p0:p0 + k] = y[at:at + k]
+            at += k
+    for s, n in enumerate(lens):
+        close(got[s], xs[s].float().double() + oracle.causal_conv(xs[s].float().double(), w), torch.float32,
+              f"x + conv(x), sequence {s}")
+
+
 # ------------------------------------------------------------------------------------------------- latent attention
 @pytest.mark.parametrize("base,rot", [(10000.0, 8), (250000.0, 16), (20.0, 2)])
 @pytest.mark.parametrize("device", ["cpu", pytest.param("cuda", marks=gpu)])
