@@ -246,6 +246,11 @@ def main():
     if dev.type == "cuda":
         torch.cuda.synchronize()
     faulthandler.cancel_dump_traceback_later()
+    # everything was stopped in order above; leave without the interpreter's own teardown, in which a daemon thread
+    # that wakes inside native code is unwound by force (seen once as "terminate called without an active exception")
+    sys.stdout.flush()
+    sys.stderr.flush()
+    os._exit(0)
 
 
 if __name__ == "__main__":
