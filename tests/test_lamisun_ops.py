@@ -332,6 +332,16 @@ def test_two_map_attention_portions_decoding_and_batches(device, dtype, H, G, d,
 
 
 @pytest.mark.parametrize("device,dtype", RUNS)
+@pytest.mark.parametrize("H,G,d,dv,chunk", [(8, 2, 64, 128, 100), (4, 4, 32, 64, 0), (6, 2, 128, 48, 128),
+                                            (3, 1, 64, 40, 77)])
+def test_two_map_attention_over_long_portions(device, dtype, H, G, d, dv, chunk):
+    """Portions of hundreds of rows beside a shorter one: many row blocks per sequence (on the matrix cores a wave
+    holds two groups of rows there), key tiles that every row of a group sees whole and tiles cut by the diagonal
+    or by a chunk's first position, a portion that continues far into its sequence."""
+    two_map_case(device, dtype, H, G, d, dv, [333, 140, 9], [[200, 133], [140], [9]], d ** -0.5, 0.45, chunk, seed=11)
+
+
+@pytest.mark.parametrize("device,dtype", RUNS)
 @pytest.mark.parametrize("d", [16, 64])
 @pytest.mark.parametrize("chunk,key,row", [(48, 96, 143), (48, 95, 143), (48, 144, 144), (48, 143, 144), (64, 128, 191),
                                            (64, 127, 191), (10, 190, 199), (10, 189, 199), (0, 0, 199), (0, 17, 199)])
