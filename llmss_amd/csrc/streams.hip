@@ -14,7 +14,7 @@
 #include "seqrows.h"
 
 #define MAX_STREAMS 8
-#define MAX_TAIL 8
+#define MAX_TAIL 16
 #define CONV_CPT 4  // channels per thread of the convolution kernel
 
 // x[s, t, :] = table[ids[t], :] (+ pos_table[positions[t], :]) for every stream s
@@ -294,7 +294,7 @@ template <typename TI, typename TW, typename TO>
 static void causal_conv_t(const void* in, int64_t ldi, const void* w, void* state, const void* cu, const void* ctx,
                           const void* sslots, void* out, int64_t ldo, int T_, int B, int C, int taps, int res,
                           int silu, hipStream_t st) {
-  if (T_ >= 256 && T_ >= 8 * B) {  // portions of eight rows and more on average
+  if (T_ >= 256 && T_ >= 8 * B && taps <= 9) {  // portions of eight rows and more on average
     const auto al16 = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
     const bool four = C % 4 == 0 && ldi % 4 == 0 && ldo % 4 == 0 && al16(in) && al16(out) && al16(state);
 #define LAUNCH_STRIP(RMAX_, CH_)                                                                                    \
@@ -304,11 +304,11 @@ static void causal_conv_t(const void* in, int64_t ldi, const void* w, void* stat
     if (four) {
       dim3 g((T_ + CONV_STRIP - 1) / CONV_STRIP, (C / 4 + 255) / 256);
       if (taps <= 4) LAUNCH_STRIP(3, 4);
-      else LAUNCH_STRIP(MAX_TAIL, 4);
+      else LAUNCH_STRIP(8, 4);
     } else {
       dim3 g((T_ + CONV_STRIP - 1) / CONV_STRIP, (C + 255) / 256);
       if (taps <= 4) LAUNCH_STRIP(3, 1);
-      else LAUNCH_STRIP(MAX_TAIL, 1);
+      else LAUNCH_STRIP(8, 1);
     }
 #undef LAUNCH_STRIP
   } else {
@@ -329,7 +329,7 @@ void launch_causal_conv(const void* in, int64_t ldi, const void* w, void* state,
                         const void* sslots, void* out, int64_t ldo, int T_, int B, int C, int taps, int res, int silu,
                         int di, int dw, int dout, hipStream_t st) {
   if (T_ == 0 || B == 0) return;
-  if (taps < 1 || taps - 1 > MAX_TAIL) throw std::runtime_error("causal_conv: 1 to 9 taps");
+  if (taps < 1 || taps - 1 > MAX_TAIL) throw std::runtime_error("causal_conv: 1 to 17 taps");
   if ((C + 255) / 256 > 65535) throw std::runtime_error("causal_conv: too many channels");
   DISPATCH_T(di, TI, DISPATCH_T(dw, TW, DISPATCH_T(dout, TO, (causal_conv_t<TI, TW, TO>(
       in, ldi, w, state, cu, ctx, sslots, out, ldo, T_, B, C, taps, res, silu, st)))));

@@ -155,7 +155,7 @@ def test_input_convolution_reads_the_fp32_residual(device, dtype, taps):
 
 
 @pytest.mark.parametrize("device,dtype", RUNS)
-@pytest.mark.parametrize("taps", [1, 2, 4, 9])
+@pytest.mark.parametrize("taps", [1, 2, 4, 9, 12])
 @pytest.mark.parametrize("C", [300, 21])
 def test_input_convolution_over_long_portions(device, dtype, taps, C):
     """Steps of several hundred rows (on a GPU the kernel that walks strips of rows): sequences of unequal length
