@@ -722,7 +722,7 @@ __global__ __launch_bounds__(256) void qk_norm_cache_kernel(const T* __restrict_
 }
 
 // The same for bf16 rows whose vectors are whole 16-byte pieces: dim / 8 neighbouring lanes (a power of two) share a
-// vector, each lane reads its eight numbers once, the sum of squares goes round the lanes of the vector, and the
+// vector, each lane reads its eight numbers once, the sum of squares is added up across the lanes of the vector, and the
 // result leaves in 16-byte stores (two for a query's eight fp32 numbers).
 __global__ __launch_bounds__(256) void qk_norm_cache_vec_kernel(const bf16_t* __restrict__ proj, int64_t ldp,
                                                                 int off_q, int off_k, int off_v,
