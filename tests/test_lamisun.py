@@ -75,7 +75,7 @@ CONFIGS = {
 
 class Case:
     def __init__(self, name, tmp, device, dtype, seed=0):
-        self.cfg = CONFIGS[name]
+        self.cfg = CONFIGS[name] if name in CONFIGS else BROAD
         mc = ModelConfig.from_hf_dict(self.cfg)
         self.sd = lamisun_state_dict(mc, seed=seed)
         d = tmp / f"{name}-{seed}"
@@ -391,6 +391,74 @@ def test_trace_runner_replays_steps_on_the_cpu_path(cases, tmp_path):
     g2 = torch.from_numpy(np.fromfile(tmp_path / "2.f32", dtype="<f4").reshape(2, c.V))
     c.close(g0, c.ref(t)[[0, 8]], "step 0")
     c.close(g2, torch.stack([c.ref(t)[20], c.ref(t[:3])[2]]), "step 2")
+
+
+# A wider model than the others here, for the GPU: rows of hundreds of tokens through the matrix-core kernels
+# (cached latent rows of 64 and 192 numbers, key sizes 32 and 64), several row blocks per portion.
+BROAD = model(700, 320, 1e-5, 2, 1.5, 257, 97, 5, [
+    lat(5, 48, 16, 48, 48, 0.12, base=5000.0, ff=640),
+    lat(10, 32, 32, 32, 160, 0.12, base=5000.0, ff=640),
+    att(10, 5, 32, 32, 0.18, 0.4, 50, ff=640),
+    att(5, 1, 64, 64, 0.125, 0.1, 512, ff=640),
+])
+
+
+@gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_runner_replays_long_requests_on_the_gpu(cases, tmp_path, dtype):
+    """bin/trace_run as a user runs it, on the GPU in both precisions: a request of 600 tokens alone in portions of
+    changing size and then token by token, then - in the pages and the slot it gave back - three requests side by
+    side, portions of some beside single tokens of others. Every position's logits against the float64 definition."""
+    import subprocess
+    import sys
+
+    c = cases("broad", "cuda", dtype)
+    reqs = {"a": toks(600, c.V, 31), "b": toks(290, c.V, 32), "c": toks(130, c.V, 33), "d": toks(5, c.V, 34)}
+    steps, at = [], {k: 0 for k in reqs}
+
+    def feed(pairs):
+        ent = []
+        for k, n in pairs:
+            ent.append(dict(id=k, tokens=reqs[k][at[k]:at[k] + n], want=list(range(n))))
+            at[k] += n
+        steps.append(dict(step=len(steps), entries=ent, end=[k for k, _ in pairs if at[k] == len(reqs[k])], rows=[
+            (k, at[k] - n + j) for k, n in pairs for j in range(n)]))
+
+    cuts = [100, 2, 133, 3, 33, 2, 17, 78, 64, 1, 1, 1, 37]
+    i = 0
+    while at["a"] < len(reqs["a"]):
+        left = len(reqs["a"]) - at["a"]
+        feed([("a", min(left, cuts[i % len(cuts)]) if left > 20 else 1)])
+        i += 1
+    pat = {"b": [150, 1, 90, 1, 1, 2], "c": [2, 1, 1, 30, 1], "d": [1, 1, 3]}
+    i = 0
+    while any(at[k] < len(reqs[k]) for k in pat):
+        pairs = [(k, min(len(reqs[k]) - at[k], pat[k][i % len(pat[k])])) for k in pat
+                 if at[k] < len(reqs[k]) and (i + ord(k)) % 5 != 4]
+        if pairs:
+            feed(pairs)
+        i += 1
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", c.path, "--dtype", dtype,
+                        "--out", str(tmp_path), "--max-tokens", "640"],
+                       input="".join(json.dumps({k: v for k, v in s.items() if k != "rows"}) + "\n" for s in steps),
+                       capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert sum(ln.startswith("done") for ln in r.stdout.splitlines()) == len(steps)
+    ref = {k: c.ref(v).double() for k, v in reqs.items()}
+    every = torch.cat(list(ref.values()))
+    spread = float((every - every.mean(-1, keepdim=True)).pow(2).mean().sqrt())
+    errs = []
+    for s in steps:
+        got = torch.from_numpy(np.fromfile(tmp_path / f"{s['step']}.f32", dtype="<f4").reshape(-1, c.V)).double()
+        want = torch.stack([ref[k][p] for k, p in s["rows"]])
+        d = (got - want) - (got - want).mean(-1, keepdim=True)
+        errs.append(d.pow(2).mean(-1).sqrt() / spread)
+    errs = torch.cat(errs)
+    if dtype == "float32":
+        assert float(errs.max()) < 5e-5, f"row {int(errs.argmax())}: {float(errs.max()):.3g} of the logits' spread"
+    else:  # bf16 products and activations: the model's own rounding noise (median 0.011, largest 0.022 of the spread)
+        assert float(errs.median()) < 0.02 and float(errs.max()) < 0.05, (float(errs.median()), float(errs.max()))
 
 
 def test_registry_facade_runs_the_design(cases):
