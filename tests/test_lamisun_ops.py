@@ -136,6 +136,11 @@ def test_xielu_and_the_output_gate(device, dtype):
     yd = y.to(dtype).to(device).clone()
     ops.gate_mul(yd, src.to(dtype).to(device), 11)
     close(yd, y * torch.sigmoid(src[:, 11:35]), dtype, "gate")
+    # rows of whole 16-byte pieces (the wide accesses of the bf16 kernel), more columns than one pass of a workgroup
+    y, src = rnd(3, 4112, seed=4, dtype=dtype), rnd(3, 4200, seed=5, dtype=dtype) * 4
+    yd = y.to(dtype).to(device).clone()
+    ops.gate_mul(yd, src.to(dtype).to(device), 88)
+    close(yd, y * torch.sigmoid(src[:, 88:]), dtype, "gate, wide rows")
 
 
 @pytest.mark.parametrize("device,dtype", RUNS)
