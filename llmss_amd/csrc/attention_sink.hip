@@ -820,10 +820,55 @@ __global__ __launch_bounds__(256) void diff_combine_kernel(const float* __restri
   }
 }
 
+// The same with vdim / 4 neighbouring lanes (a power of two) to a head: each lane reads its four numbers of both
+// maps in 16-byte pieces once and writes its four results in one piece.
+template <typename T>
+__global__ __launch_bounds__(256) void diff_combine_vec_kernel(const float* __restrict__ O, float lam, float eps,
+                                                               float mult, T* __restrict__ y, int64_t ldy, int H,
+                                                               int G, int vdim) {
+  const int t = blockIdx.x;
+  const int L = vdim >> 2, sub = threadIdx.x & (L - 1), per = blockDim.x / L;
+  const int rep = H / G;
+  for (int h = blockIdx.y * per + threadIdx.x / L; h < H; h += gridDim.y * per) {
+    const int g = h / rep, r = h - g * rep;
+    const float* a1 = O + ((int64_t)t * 2 * H + (g * 2) * rep + r) * vdim + 4 * sub;
+    const f32x4 x1 = *reinterpret_cast<const f32x4*>(a1);
+    const f32x4 x2 = *reinterpret_cast<const f32x4*>(a1 + (int64_t)rep * vdim);
+    float o[4];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      o[i] = x1[i] - lam * x2[i];
+      ss = fmaf(o[i], o[i], ss);
+    }
+    for (int d = L >> 1; d > 0; d >>= 1) ss += __shfl_xor(ss, d, 64);
+    const float inv = mult / sqrtf(ss / (float)vdim + eps);
+    T* dst = y + (int64_t)t * ldy + (int64_t)h * vdim + 4 * sub;
+    if constexpr (sizeof(T) == 4) {
+      *reinterpret_cast<f32x4*>(dst) = f32x4{o[0] * inv, o[1] * inv, o[2] * inv, o[3] * inv};
+    } else {
+      u32x2 pk;
+      pk[0] = (unsigned)f2bf(o[0] * inv) | ((unsigned)f2bf(o[1] * inv) << 16);
+      pk[1] = (unsigned)f2bf(o[2] * inv) | ((unsigned)f2bf(o[3] * inv) << 16);
+      *reinterpret_cast<u32x2*>(dst) = pk;
+    }
+  }
+}
+
 void launch_diff_combine(const void* O, float lam, float eps, float mult, void* y, int64_t ldy, int T_, int H, int G,
                          int vdim, int dt, hipStream_t st) {
   if (T_ == 0) return;
   if (G < 1 || H % G) throw std::runtime_error("diff_combine: heads must be a multiple of the key heads");
+  const int L = vdim / 4;
+  if (vdim % 4 == 0 && L >= 1 && L <= 64 && (L & (L - 1)) == 0 && ldy % 4 == 0 && ((uintptr_t)O & 15) == 0 &&
+      ((uintptr_t)y & 15) == 0) {
+    const int per = 256 / L;
+    dim3 g(T_, std::min(64, (H + per - 1) / per));
+    DISPATCH_T(dt, T, (diff_combine_vec_kernel<T><<<g, 256, 0, st>>>((const float*)O, lam, eps, mult, (T*)y, ldy, H,
+                                                                      G, vdim)));
+    HIP_CHECK_LAUNCH();
+    return;
+  }
   dim3 g(T_, std::min(64, (H + 3) / 4));
   DISPATCH_T(dt, T, (diff_combine_kernel<T><<<g, 256, 0, st>>>((const float*)O, lam, eps, mult, (T*)y, ldy, H, G,
                                                                 vdim)));
