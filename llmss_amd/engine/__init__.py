@@ -9,9 +9,10 @@ import torch
 from ..models.config import ModelConfig, get_preset
 from ..models.decoder import DecoderLM
 from ..models.layered import LayeredLM, create_model
-from ..models.weights import (load_babotar_weights, load_hf_weights, load_lamisun_weights, load_shard,
-                              load_timisun_weights, random_babotar_weights, random_lamisun_weights,
-                              random_timisun_weights, random_weights, save_shard, shard_cache_path)
+from ..models.weights import (load_babotar_weights, load_fizelix_weights, load_hf_weights, load_lamisun_weights,
+                              load_shard, load_timisun_weights, random_babotar_weights, random_fizelix_weights,
+                              random_lamisun_weights, random_timisun_weights, random_weights, save_shard,
+                              shard_cache_path)
 from ..parallel.dist import TPGroup
 from ..utils.checkpoint import CheckpointReader, weight_files
 from .engine import LLMEngine, Request, StepEvent
@@ -50,7 +51,8 @@ def build_model(model: str, tp: Optional[TPGroup] = None, dtype: str = "bf16", d
         if fp8:
             raise ValueError(f"{cfg.model_type}: fp8 weights are not supported")
         rand, load = {"babotar": (random_babotar_weights, load_babotar_weights),
-                      "lamisun": (random_lamisun_weights, load_lamisun_weights)}.get(
+                      "lamisun": (random_lamisun_weights, load_lamisun_weights),
+                      "fizelix": (random_fizelix_weights, load_fizelix_weights)}.get(
             cfg.model_type, (random_timisun_weights, load_timisun_weights))
         if random_init:
             w = rand(cfg, device=device, dtype=tdtype, seed=seed)

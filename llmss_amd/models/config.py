@@ -28,6 +28,13 @@ Families (``MODEL_REGISTRY`` keys, reference ``custom_modeling/__init__.py:4-7``
                     embedding; mixers ``latent_attention`` (with a rotated key part shared by the heads and an output
                     gate) and ``attention`` (two softmax maps subtracted, chunked mask, query / key norm);
                     plain feed-forward with the xIELU activation, untied head.
+* ``fizelix``     - per-layer description: blocks normed before AND after each sublayer, the sublayer's result gated
+                    by sigmoid(W h + b) and scaled per channel, a per-layer token input after the feed-forward, a run
+                    of layers repeated with the same weights (the embedding added again before each repeat); mixers
+                    ``pool_attention`` (sigmoid-weighted sliding window plus mean-pooled blocks of older tokens,
+                    neighbour-pair rotation) and ``mamba2`` (state-space duality: decayed matrix state per head, short
+                    convolution, gate before a grouped norm); feed-forward dense SiLU-gated or mixture of experts whose
+                    sigmoid score multiplies the expert's input; scaled logits, untied head.
 """
 from __future__ import annotations
 
@@ -64,7 +71,7 @@ class MixerSpec:
 @dataclass
 class ExpertSpec:
     ff: int
-    limit: float
+    limit: float = 0.0
 
 
 @dataclass
@@ -76,6 +83,9 @@ class MoESpec:
     expert: ExpertSpec
     shared: Optional[ExpertSpec] = None
     kind: str = "moe"
+    act: str = "glu_clamp"  # "glu_clamp": g sigmoid(1.702 g) (u + 1) with clamps; "silu": silu(g) u, no clamps
+    normalize: bool = True  # the chosen scores are divided by their sum
+    weight_input: bool = False  # the score multiplies the expert's input (sum_e expert_e(w_e h)), not its output
 
 
 @dataclass
@@ -124,6 +134,47 @@ class DiffAttnSpec:
     chunk: int = 0
     qk_norm: bool = True
     kind: str = "attention"
+
+
+@dataclass
+class PoolAttnSpec:
+    """Sigmoid-weighted attention over a paged key/value cache, no softmax: ``heads`` query heads on ``kv_heads``
+    key/value heads; the weight of a visible key is sigmoid(q . k * scale + bias[head]), weights are not normalised.
+    Position i sees the positions j with 0 <= i - j < ``window`` (0: all earlier ones) and, with ``pool`` > 0, one
+    mean key and mean value for every block of ``pool`` positions that ends at or before i - window. ``rot``:
+    rotation of neighbouring pairs of the first ``rot.dims`` numbers of every query and key head."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    window: int = 0
+    pool: int = 0
+    rot: Optional[RotarySpec] = None
+    kind: str = "pool_attention"
+
+
+@dataclass
+class SSDSpec:
+    """State-space mixer with a scalar decay per head and token: a matrix state [state, vdim] per head, ``groups``
+    input / output vectors (B, C) shared by heads / groups heads each, x | B | C through a causal convolution of
+    ``conv`` taps with bias and SiLU; the heads' outputs are gated by silu(z) and then RMS-normed in ``norm_groups``
+    equal parts."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int = 1
+    kind: str = "mamba2"
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
 
 
 @dataclass
@@ -227,6 +278,21 @@ class ModelConfig:
     canon_ffn: bool = False  # the feed-forward's input goes through an input convolution of its own as well
     depth_average: bool = False  # what leaves layer i is a learned weighted sum of the results of layers <= i
     bigram: Optional[BigramSpec] = None
+    # blocks normed on both sides of a sublayer: x <- x + scale * norm_b(gate * sublayer(norm_a(x))), gate =
+    # sigmoid(W norm_a(x) + b) per channel
+    sandwich: bool = False
+    token_side_dim: int = 0  # > 0: after the feed-forward a layer adds a normed projection of its slice of a second token table
+    loop: Optional[tuple] = None  # (start, stop, times): layers start .. stop - 1 run ``times`` times in a row
+    logit_scale: float = 1.0
+
+    def layer_runs(self) -> List[int]:
+        """Layer index of every layer run, in order: a looped stretch repeats with the same weights, each pass with
+        cache and state of its own."""
+        n = len(self.layer_specs) if self.layer_specs else self.num_layers
+        if not self.loop or self.loop[2] <= 1:
+            return list(range(n))
+        a, b, times = self.loop
+        return list(range(a)) + list(range(a, b)) * times + list(range(b, n))
 
     # ---------------------------------------------------------------- derived
     @property
@@ -247,10 +313,11 @@ class ModelConfig:
 
     def num_params(self) -> int:
         h, f, v = self.hidden_size, self.intermediate_size, self.vocab_size
-        if self.layer_specs and self.model_type in ("babotar", "lamisun"):
-            from .weights import babotar_shapes, lamisun_shapes
+        if self.layer_specs and self.model_type in ("babotar", "lamisun", "fizelix"):
+            from .weights import babotar_shapes, fizelix_shapes, lamisun_shapes
 
-            shapes = babotar_shapes(self) if self.model_type == "babotar" else lamisun_shapes(self)
+            shapes = {"babotar": babotar_shapes, "lamisun": lamisun_shapes, "fizelix": fizelix_shapes}[
+                self.model_type](self)
             return sum(math.prod(shp) for shp in shapes.values())
         if self.layer_specs:
             n = v * h + h
@@ -282,6 +349,8 @@ class ModelConfig:
             return _babotar(cls, d)
         if mt is None and d.get("architecture") == "Lamisun":
             return _lamisun(cls, d)
+        if mt is None and d.get("architecture") == "Fizelix":
+            return _fizelix(cls, d)
         common = dict(
             bos_token_id=d.get("bos_token_id"),
             eos_token_id=_first(d.get("eos_token_id")),
@@ -499,6 +568,75 @@ def _lamisun(cls, d: Dict[str, Any]) -> "ModelConfig":
     )
 
 
+def _fizelix(cls, d: Dict[str, Any]) -> "ModelConfig":
+    """``{"architecture": "Fizelix", "vocab", "width", "norm": {"eps"}, "embedding": {"scale"}, "logit_scale",
+    "token_side": {"dim"}, "loop": {"start", "stop", "times"}, "layers": [{"type": "attention" | "mamba2", "mixer":
+    {...}, "mlp": {"kind": "dense", "ff"} | {"kind": "moe", "router": {"experts", "top"}, "expert": {"ff"}, "shared":
+    {"ff"}} | null}]}``. An attention mixer gives heads, kv_heads, dim, vdim, scale, mask: {size, pool}, rot: {base,
+    dims}; a mamba2 mixer heads, vdim, state, groups, conv, norm_groups. Keys a config leaves out switch their
+    mechanism off (no loop, no token input, no rotation, no pooled blocks, no window, no shared expert)."""
+    specs: List[LayerSpec] = []
+    for i, L in enumerate(d["layers"]):
+        m, typ = L["mixer"], L.get("type")
+        if typ == "attention":
+            rot = None
+            if m.get("rot") and int(m["rot"].get("dims") or 0):
+                rot = RotarySpec(int(m["rot"]["dims"]), float(m["rot"]["base"]), None, "neighbours")
+                if rot.dims % 2 or rot.dims > int(m["dim"]):
+                    raise ValueError(f"Fizelix layer {i}: {rot.dims} rotary dimensions on heads of {m['dim']}")
+            mask = m.get("mask") or {}
+            mixer = PoolAttnSpec(int(m["heads"]), int(m.get("kv_heads") or m["heads"]), int(m["dim"]), int(m["vdim"]),
+                                 float(m["scale"]), int(mask.get("size") or 0), int(mask.get("pool") or 0), rot)
+            if mixer.heads % mixer.kv_heads:
+                raise ValueError(f"Fizelix layer {i}: {mixer.heads} heads on {mixer.kv_heads} key heads")
+            if mixer.pool and not mixer.window:
+                raise ValueError(f"Fizelix layer {i}: pooled blocks need a window")
+        elif typ == "mamba2":
+            mixer = SSDSpec(int(m["heads"]), int(m["vdim"]), int(m["state"]), int(m.get("groups") or 1),
+                            int(m.get("conv") or 1), int(m.get("norm_groups") or 1))
+            if mixer.heads % mixer.groups or mixer.inner % mixer.norm_groups:
+                raise ValueError(f"Fizelix layer {i}: {mixer.heads} heads in {mixer.groups} groups, "
+                                 f"{mixer.inner} channels in {mixer.norm_groups} norm groups")
+        else:
+            raise ValueError(f"Fizelix layer {i}: unsupported mixer type {typ!r}")
+        f, mlp = L.get("mlp"), None
+        if f is not None:
+            kind = f.get("kind", "dense")
+            if kind == "dense":
+                mlp = DenseMLPSpec(int(f["ff"]), "silu")
+            elif kind == "moe":
+                sh = f.get("shared")
+                mlp = MoESpec(int(f["router"]["experts"]), int(f["router"]["top"]), ExpertSpec(int(f["expert"]["ff"])),
+                              None if not sh else ExpertSpec(int(sh["ff"])), act="silu", normalize=False,
+                              weight_input=True)
+                if not 1 <= mlp.top <= mlp.experts:
+                    raise ValueError(f"Fizelix layer {i}: top {mlp.top} of {mlp.experts} experts")
+            else:
+                raise ValueError(f"Fizelix layer {i}: unsupported feed-forward kind {kind!r}")
+        specs.append(LayerSpec(mixer, mlp))
+    if not specs:
+        raise ValueError("Fizelix: no layers")
+    loop = None
+    lp = d.get("loop")
+    if lp and int(lp.get("times", 1)) > 1:
+        loop = (int(lp["start"]), int(lp["stop"]), int(lp["times"]))
+        if not 0 <= loop[0] < loop[1] <= len(specs):
+            raise ValueError(f"Fizelix: loop over layers {loop[0]} .. {loop[1] - 1} of {len(specs)}")
+    ffs = [s.mlp.ff if s.mlp.kind == "dense" else s.mlp.expert.ff for s in specs if s.mlp]
+    return cls(
+        model_type="fizelix", vocab_size=int(d["vocab"]), hidden_size=int(d["width"]), num_layers=len(specs),
+        num_heads=max(s.mixer.heads for s in specs), num_kv_heads=1, head_dim=1, intermediate_size=max(ffs or [0]),
+        max_position_embeddings=1 << 20,  # the design has no positional limit of its own
+        norm="rmsnorm", norm_eps=float(d["norm"]["eps"]), activation="silu_glu", position="none", rotary_dim=0,
+        parallel_block=False, tie_word_embeddings=False, layer_specs=specs, residual_fp32=True,
+        embedding_scale=float((d.get("embedding") or {}).get("scale", 1.0)), sandwich=True,
+        token_side_dim=int((d.get("token_side") or {}).get("dim") or 0), loop=loop,
+        logit_scale=float(d.get("logit_scale", 1.0)),
+        bos_token_id=d.get("bos_token_id"), eos_token_id=_first(d.get("eos_token_id")),
+        pad_token_id=d.get("pad_token_id"),
+    )
+
+
 def _first(x):
     if isinstance(x, (list, tuple)):
         return x[0] if x else None
@@ -604,6 +742,22 @@ _PRESETS: Dict[str, Dict[str, Any]] = {
                                   mixer=dict(heads=2, dim=8, rot_dim=4, vdim=16, kv_rank=20, scale=0.3,
                                              rot=dict(base=10000.0, dims=4)),
                                   mlp=dict(kind="dense", ff=64)),
+                         ]),
+    # sandwich-normed per-layer design: windowed sigmoid attention with pooled blocks, a state-space layer, dense and
+    # expert feed-forwards, a looped stretch, token input
+    "tiny-fizelix": dict(architecture="Fizelix", vocab=211, width=48, norm=dict(eps=1e-5), embedding=dict(scale=2.0),
+                         logit_scale=0.5, token_side=dict(dim=6), loop=dict(start=1, stop=3, times=2),
+                         layers=[
+                             dict(type="mamba2",
+                                  mixer=dict(heads=4, vdim=12, state=8, groups=2, conv=4, norm_groups=2),
+                                  mlp=dict(kind="dense", ff=64)),
+                             dict(type="attention",
+                                  mixer=dict(heads=4, kv_heads=2, dim=8, vdim=12, scale=0.3,
+                                             mask=dict(size=7, pool=3), rot=dict(base=1000.0, dims=4)),
+                                  mlp=dict(kind="moe", router=dict(experts=5, top=2), expert=dict(ff=20),
+                                           shared=dict(ff=12))),
+                             dict(type="mamba2",
+                                  mixer=dict(heads=3, vdim=16, state=12, groups=1, conv=2, norm_groups=1), mlp=None),
                          ]),
     # TP up to 8 (16 q / kv heads: 2 per rank at TP=8, as Llama-2-7B's 32 give 4)
     "tiny-llama16h": dict(model_type="llama", hidden_size=256, num_hidden_layers=2, num_attention_heads=16,

@@ -1,7 +1,7 @@
 """Decoder whose layers are described one by one (``ModelConfig.layer_specs``) over an fp32 residual stream.
 
 The uniform families run through :class:`~llmss_amd.models.decoder.DecoderLM`; a per-layer design (Timisun, Babotar,
-Lamisun) runs through :class:`LayeredLM`, which offers the engine the same surface (``hidden_states`` / ``logits`` over a
+Lamisun, Fizelix) runs through :class:`LayeredLM`, which offers the engine the same surface (``hidden_states`` / ``logits`` over a
 :class:`StepInput`, ``allocate_kv_cache``, ``kv_bytes_per_block``, ``plan``) and so shares its scheduler, paged
 cache pool, decode graphs and sampler. A layer is either a parallel block (``cfg.parallel_block``)
 
@@ -17,7 +17,14 @@ on each sublayer's output,
     x <- x + norm1(mixer(x + conv1(x))) ;  x <- x + norm2(ffn(x + conv2(x)))
 
 optionally followed by a depth average: what goes on to the next layer is sum_j dwa[j] X_j over the results X_j of
-this and all earlier layers (X_0 the embedding). The mixer and the feed-forward are looked up by kind
+this and all earlier layers (X_0 the embedding); or (``cfg.sandwich``) a sequential block normed on both sides of
+each sublayer, its result gated per channel and scaled,
+
+    h = norm_a(x) ;  x <- x + post * rms_norm(sigmoid(W_g h + b) * sublayer(h))          post = norm_b weight * layer scale
+
+optionally followed by a token input (x <- x + rms_norm(W_p (gelu(W_s x) * e)) * w, e the layer's slice of a second
+token table); a stretch of such layers may run several times in a row with the same weights (``cfg.loop``), each pass
+with cache and state of its own, the embedding added again before every pass but the first. The mixer and the feed-forward are looked up by kind
 (``MIXERS`` / ``FFNS``), so another design can combine the same mechanisms with other constants or add its own
 beside them. Besides pages of the shared pool a mixer may own per-sequence state (a matrix state per head, the last
 inputs of a convolution): ``LayerCache.state`` tensors indexed by the scheduler's state slot of each sequence
@@ -43,9 +50,16 @@ and keys and a chunked causal mask. The two maps of a key head are cached as two
 heads of a group are laid out so that the grouped-query kernel's head mapping serves them (``vshare`` = 2: both key
 heads read one value head).
 
+Mixer ``pool_attention`` (ops: linear_f, rope_angles, rope_pairs_cache, pool_update, pool_window_attn): grouped-query
+attention without a softmax - a visible key weighs sigmoid(score + bias_h) - over a sliding window and, beyond it,
+one mean key / value per block of ``pool`` positions that has wholly left the window; the means live in a pooled cache
+beside the pages (one row per block, written when the block's last position is). Mixer ``mamba2`` (causal_conv with
+bias, ssd_recurrence, gated_group_norm gate-first): S <- exp(-exp(A) dt) S + dt B x^T, y = S^T C + D x per head.
+
 Feed-forward ``moe`` (ops: moe_router -> fp32 router logits and routing, moe_experts, glu_clamp): sigmoid scores, the
 choice made on score + correction, weights = chosen scores normalised; experts and the shared expert use the clamped
-gated activation g * sigmoid(1.702 g) * (u + 1).
+gated activation g * sigmoid(1.702 g) * (u + 1); or, by the spec, unnormalised scores that multiply the expert's
+INPUT and plain silu(g) * u.
 """
 from __future__ import annotations
 
@@ -138,14 +152,18 @@ class MoEFeedForward:
     @staticmethod
     def forward(model: "LayeredLM", W, spec, h):
         dt = model.dtype
-        idx, wts = ops.moe_router(h, W.router, W.correction, spec.top)
+        idx, wts = ops.moe_router(h, W.router, W.correction, spec.top, spec.normalize)
         sh = None
         if W.shared_gu is not None:
-            gu = ops.linear_f(h, W.shared_gu, dt)
-            sh = ops.linear_f(ops.glu_clamp(gu, spec.shared.ff, spec.shared.limit, GLU_ALPHA), W.shared_down, dt)
+            # (a sandwich block's gate logits ride in this GEMM as extra columns: model.proj)
+            gu = model.proj = ops.linear_f(h, W.shared_gu, dt)
+            if spec.shared is not None:
+                a = ops.glu_act(gu, spec.shared.ff, "silu") if spec.act == "silu" else \
+                    ops.glu_clamp(gu, spec.shared.ff, spec.shared.limit, GLU_ALPHA)
+                sh = ops.linear_f(a, W.shared_down, dt)
         # combine=False: on the GPU the weighted sum over the chosen experts happens inside the next residual add
         return ops.moe_experts(h, idx, wts, W.gate, W.up, W.down, spec.expert.limit, GLU_ALPHA, shared=sh,
-                               combine=False)
+                               combine=False, act=spec.act, weight_input=spec.weight_input)
 
 
 class ParallelMixer:
@@ -238,11 +256,94 @@ class DenseFeedForward:
         dt = model.dtype
         if not spec.gated:
             return ops.linear_f(ops.act_fn(ops.linear_f(h, W.gu, dt), spec.act, W.act_params), W.down, dt)
-        return ops.linear_f(ops.glu_act(ops.linear_f(h, W.gu, dt), spec.ff, spec.act), W.down, dt)
+        gu = model.proj = ops.linear_f(h, W.gu, dt)  # (columns past 2 ff: a sandwich block's gate logits)
+        return ops.linear_f(ops.glu_act(gu, spec.ff, spec.act), W.down, dt)
+
+
+class PoolAttention:
+    """Mixer ``pool_attention``: sigmoid-weighted grouped-query attention over a sliding window of the paged key /
+    value rows plus one mean row per block of ``pool`` positions behind the window."""
+
+    @staticmethod
+    def cache_row(spec) -> Optional[int]:
+        return spec.kv_heads * (spec.dim + spec.vdim)
+
+    @staticmethod
+    def pooled_per_page(spec, block_size: int) -> int:
+        return -(-block_size // spec.pool) if spec.pool else 0
+
+    @staticmethod
+    def allocate(model: "LayeredLM", spec, num_blocks: int, block_size: int, num_slots: int):
+        dt, dev = model.dtype, model.device
+        per = PoolAttention.pooled_per_page(spec, block_size)
+        pooled = {}
+        if per:  # fp32 means, row (page of the block's first position, rank of the block among those starting there)
+            pooled = {"kp": torch.zeros(num_blocks, per, spec.kv_heads * spec.dim, dtype=torch.float32, device=dev),
+                      "vp": torch.zeros(num_blocks, per, spec.kv_heads * spec.vdim, dtype=torch.float32, device=dev)}
+        return (torch.zeros(num_blocks, block_size, spec.kv_heads * spec.dim, dtype=dt, device=dev),
+                torch.zeros(num_blocks, block_size, spec.kv_heads * spec.vdim, dtype=dt, device=dev), pooled)
+
+    @staticmethod
+    def extra_bytes_per_block(spec, block_size: int) -> int:
+        return 4 * PoolAttention.pooled_per_page(spec, block_size) * spec.kv_heads * (spec.dim + spec.vdim)
+
+    @staticmethod
+    def forward(model: "LayeredLM", i: int, W, spec, h, inp: StepInput, cu, caches):
+        dt, c = model.dtype, W.cols
+        kc, vc, pooled = caches[i]
+        proj = model.proj = ops.linear_f(h, W.proj, dt)
+        cs = model.angles(inp, W.rot_key, W.freqs) if W.freqs is not None else None
+        q = ops.rope_pairs_cache(proj, c["q"], c["k"], c["v"], cs, kc, vc, inp.slots, spec.heads, spec.kv_heads,
+                                 spec.dim, spec.vdim)
+        kp, vp = pooled.get("kp"), pooled.get("vp")
+        if spec.pool:
+            ops.pool_update(kc, vc, kp, vp, inp.block_tables, cu, inp.ctx_lens, spec.pool)
+        single = inp.kind == "decode"
+        y = ops.pool_window_attn(q, kc, vc, kp, vp, inp.block_tables, cu, inp.ctx_lens, W.pb, spec.heads,
+                                 spec.kv_heads, spec.dim, spec.vdim, spec.scale, spec.window, spec.pool, dt,
+                                 max_qlen=1 if single else max(1, inp.max_seqlen),
+                                 num_decode=0 if single else inp.num_decode)
+        return ops.linear_f(y, W.o, dt)
+
+
+class SSDMixer:
+    """Mixer ``mamba2``: x | B | C through a short causal convolution with bias and SiLU, the scalar-decay state-space
+    recurrence over a matrix state per head, the result gated by silu(z) and then normed in groups."""
+
+    @staticmethod
+    def cache_row(spec) -> Optional[int]:
+        return None
+
+    @staticmethod
+    def allocate(model: "LayeredLM", spec, num_blocks: int, block_size: int, num_slots: int):
+        dev = model.device
+        return (None, None,
+                {"S": torch.zeros(num_slots, spec.heads, spec.state, spec.vdim, dtype=torch.float32, device=dev),
+                 "tail": torch.zeros(num_slots, max(spec.conv - 1, 0), spec.conv_channels, dtype=torch.float32,
+                                     device=dev)})
+
+    @staticmethod
+    def state_bytes(spec) -> int:
+        return 4 * (spec.heads * spec.state * spec.vdim + max(spec.conv - 1, 0) * spec.conv_channels)
+
+    @staticmethod
+    def forward(model: "LayeredLM", i: int, W, spec, h, inp: StepInput, cu, caches):
+        dt, c = model.dtype, W.cols
+        st = caches[i][2]
+        inner, gn = spec.inner, spec.groups * spec.state
+        proj = model.proj = ops.linear_f(h, W.proj, dt)
+        xbc = ops.causal_conv(proj[:, c["xbc"]:c["xbc"] + spec.conv_channels], W.conv, st["tail"], cu, inp.ctx_lens,
+                              inp.state_slots, False, True, dt, bias=W.conv_b)
+        y = ops.ssd_recurrence(xbc[:, :inner], xbc[:, inner:inner + gn], xbc[:, inner + gn:],
+                               proj[:, c["dt"]:c["dt"] + spec.heads], W.A_log, W.dt_bias, W.D, st["S"], cu,
+                               inp.ctx_lens, inp.state_slots, spec.heads, spec.groups, spec.state, spec.vdim)
+        y = ops.gated_group_norm(y, proj[:, c["z"]:c["z"] + inner], W.norm, model.cfg.norm_eps, "silu", 1.0,
+                                 out_dtype=dt, groups=spec.norm_groups, gate_first=True)
+        return ops.linear_f(y, W.o, dt)
 
 
 MIXERS = {"latent_attention": LatentAttention, "parallel": ParallelMixer, "lightning": DecayMixer,
-          "attention": DiffAttention}
+          "attention": DiffAttention, "pool_attention": PoolAttention, "mamba2": SSDMixer}
 FFNS = {"moe": MoEFeedForward, "dense": DenseFeedForward}
 
 
@@ -273,7 +374,8 @@ class LayeredLM:
         self.gqa_mfma: set = set()
         self._cu_decode = {}
         self._angles = {}
-        self.tap = None  # tap(i, x): called with the fp32 residual after layer i (debugging, tests)
+        self.tap = None  # tap(i, x): called with the fp32 residual after layer (run) i (debugging, tests)
+        self.proj = None  # the last sublayer's first GEMM output (a sandwich block reads its gate logits there)
 
     @property
     def device(self):
@@ -305,17 +407,25 @@ class LayeredLM:
                 if hasattr(L.mix, nm):
                     put(nm, getattr(L.mix, nm))
             for nm in ("shared_gu", "shared_down", "gu", "down"):
-                if L.mlp is not None and getattr(L.mlp, nm, None) is not None and getattr(L.mlp, nm).dim() == 2:
+                if getattr(L, "mlp", None) is not None and getattr(L.mlp, nm, None) is not None and \
+                        getattr(L.mlp, nm).dim() == 2:
                     put(nm, getattr(L.mlp, nm))
         put("head", self.w.head.w)
         return out
 
     # --------------------------------------------------------------------------------- cache
+    def _run_specs(self):
+        """The spec of every layer RUN (a looped stretch repeats): caches and state are per run."""
+        return [self.cfg.layer_specs[i] for i in self.cfg.layer_runs()]
+
     def _cache_rows(self) -> List[Optional[int]]:
-        return [MIXERS[s.mixer.kind].cache_row(s.mixer) for s in self.cfg.layer_specs]
+        return [MIXERS[s.mixer.kind].cache_row(s.mixer) for s in self._run_specs()]
 
     def kv_bytes_per_block(self, block_size: int) -> int:
-        return max(1, sum(block_size * r * self.w.wte.element_size() for r in self._cache_rows() if r))
+        n = sum(block_size * r * self.w.wte.element_size() for r in self._cache_rows() if r)
+        n += sum(MIXERS[s.mixer.kind].extra_bytes_per_block(s.mixer, block_size) for s in self._run_specs()
+                 if hasattr(MIXERS[s.mixer.kind], "extra_bytes_per_block"))
+        return max(1, n)
 
     @property
     def needs_state(self) -> bool:
@@ -327,20 +437,20 @@ class LayeredLM:
         return 2 if self.cfg.canon_ffn else 1
 
     def state_bytes_per_slot(self) -> int:
-        n = sum(MIXERS[s.mixer.kind].state_bytes(s.mixer) for s in self.cfg.layer_specs
+        n = sum(MIXERS[s.mixer.kind].state_bytes(s.mixer) for s in self._run_specs()
                 if hasattr(MIXERS[s.mixer.kind], "state_bytes"))
         n += 8 if self.cfg.bigram is not None else 0
         return n + 4 * max(self.cfg.canon_taps - 1, 0) * self.cfg.hidden_size * len(self.cfg.layer_specs) * \
             self._canon_sublayers()
 
     def allocate_kv_cache(self, num_blocks: int, block_size: int, num_slots: int = 0):
-        """One entry per layer. Latent attention: (rows, None), a layer that reads another layer's rows holding that
+        """One entry per layer run (a looped stretch of layers has an entry per pass). Latent attention: (rows, None), a layer that reads another layer's rows holding that
         layer's pair. Mixers with an ``allocate`` of their own: (key pages, value pages, {name: per-slot state});
         ``num_slots`` state slots, one per running sequence. The input convolution's tails of all layers live in
         ``self.canon_tail`` [layers (x 2 when the feed-forward has a convolution too: mixer, feed-forward), slots,
         taps - 1, W], the token before each sequence's next one (bigram embedding) in ``self.prev_token`` [slots]."""
         caches: list = []
-        for s, r in zip(self.cfg.layer_specs, self._cache_rows()):
+        for s, r in zip(self._run_specs(), self._cache_rows()):
             mx = MIXERS[s.mixer.kind]
             if hasattr(mx, "allocate"):
                 if num_slots <= 0 and hasattr(mx, "state_bytes"):
@@ -379,6 +489,8 @@ class LayeredLM:
         if inp.block_tables is None or inp.ctx_lens is None or not any(t is not None for t in kv_caches[0]):
             raise ValueError(f"{self.cfg.model_type} attends through its paged cache: the step needs block tables, "
                              f"context lengths and a cache (a cache-less recompute step is not supported)")
+        if self.cfg.sandwich:
+            return self._sandwich_blocks(inp, kv_caches)
         if self.cfg.post_norm:
             return self._postnorm_blocks(inp, kv_caches)
         if not self.cfg.parallel_block:
@@ -475,6 +587,54 @@ class LayeredLM:
                 self.tap(i, x)
         self._angles = {}
         return ops.resid_add_norm(x, None, None, w.lnf_w, 0.0, eps, dt)
+
+    def _sandwich_blocks(self, inp: StepInput, kv_caches) -> torch.Tensor:
+        """Blocks normed on both sides of their sublayers. Every sublayer's closing op (the gated, normed, scaled
+        residual add, or the token input after it) also forms what the next reader takes - the next sublayer's normed
+        input, with the embedding added first where a new pass of a looped stretch begins - as the residual add and
+        the next norm are one op for the other families. The gate logits come out of the sublayer's own first GEMM
+        (``self.proj``). With a ``tap`` the closing ops run unfused, so that the tap sees the residual as the layer
+        leaves it."""
+        cfg, w, dt = self.cfg, self.w, self.dtype
+        if self.needs_state and inp.state_slots is None:
+            raise ValueError(f"{cfg.model_type} keeps per-sequence state: the step needs the sequences' state slots")
+        eps = cfg.norm_eps
+        cu = self._cu(inp)
+        self._angles = {}
+        runs = cfg.layer_runs()
+        x = ops.embed_scaled(inp.input_ids, w.wte, cfg.embedding_scale)
+        x0 = x.clone() if cfg.loop else None
+        W_ = cfg.hidden_size
+        h = ops.sandwich_add_norm(x, None, None, None, None, eps, None, w.layers[runs[0]].norm1, dt)
+        for r, i in enumerate(runs):
+            L, spec = w.layers[i], cfg.layer_specs[i]
+            last = r + 1 == len(runs)
+            nxt = w.lnf_w if last else w.layers[runs[r + 1]].norm1
+            # the embedding comes back in before a pass of the looped stretch other than the first
+            add = x0 if not last and cfg.loop and runs[r + 1] == cfg.loop[0] and r + 1 > cfg.loop[0] else None
+            if self.tap is not None:
+                tail = (None, None)  # close the layer first, tap, then add / norm on their own
+            else:
+                tail = (add, nxt)
+            side = L.side_gate is not None
+            y = MIXERS[spec.mixer.kind].forward(self, r, L.mix, spec.mixer, h, inp, cu, kv_caches)
+            c0 = L.mix.cols["rg"]
+            after = (None, L.norm2) if spec.mlp is not None else ((None, None) if side else tail)
+            h = ops.sandwich_add_norm(x, y, self.proj[:, c0:c0 + W_], L.rg1_b, L.post1, eps, *after, dt)
+            if spec.mlp is not None:
+                y = FFNS[spec.mlp.kind].forward(self, L.mlp, spec.mlp, h)
+                after = (None, None) if side else tail
+                h = ops.sandwich_add_norm(x, y, self.proj[:, L.rg2_col:L.rg2_col + W_], L.rg2_b, L.post2, eps, *after,
+                                          dt)
+            if side:
+                h = ops.token_side_add(x, inp.input_ids, w.extra["side"], L.side_col, L.side_gate, L.side_proj,
+                                       L.side_norm, eps, *tail, dt)
+            if self.tap is not None:
+                self.tap(r, x)
+                h = ops.sandwich_add_norm(x, None, None, None, None, eps, add, nxt, dt)
+        self._angles = {}
+        self.proj = None
+        return h
 
     @property
     def vocab_lo(self) -> int:

@@ -21,7 +21,8 @@ from ..parallel.dist import TPGroup
 from .config import ModelConfig
 from .decoder import StepInput
 from .layered import create_model
-from .weights import load_babotar_weights, load_hf_weights, load_lamisun_weights, load_timisun_weights
+from .weights import (load_babotar_weights, load_fizelix_weights, load_hf_weights, load_lamisun_weights,
+                      load_timisun_weights)
 
 
 @dataclass
@@ -54,9 +55,9 @@ class CausalLM:
     def __init__(self, config, weights, max_blocks: int = 4096, block_size: int = 16, max_seqs: int = 16):
         cfg = config if isinstance(config, ModelConfig) else ModelConfig.from_hf_dict(config.to_dict())
         tp = getattr(weights, "tp", None) or TPGroup()
-        if cfg.layer_specs:  # per-layer designs (Timisun, Babotar, Lamisun)
-            load = {"babotar": load_babotar_weights, "lamisun": load_lamisun_weights}.get(cfg.model_type,
-                                                                                          load_timisun_weights)
+        if cfg.layer_specs:  # per-layer designs (Timisun, Babotar, Lamisun, Fizelix)
+            load = {"babotar": load_babotar_weights, "lamisun": load_lamisun_weights,
+                    "fizelix": load_fizelix_weights}.get(cfg.model_type, load_timisun_weights)
             w = load(cfg, weights.reader, device=weights.device, dtype=weights.dtype)
         else:
             w = load_hf_weights(cfg, weights.reader, tp.size, tp.rank, device=weights.device, dtype=weights.dtype)
@@ -283,6 +284,13 @@ class LamisunForCausalLM(_FamilyLM):
     model_type = "lamisun"
 
 
+class FizelixForCausalLM(_FamilyLM):
+    """Per-layer design: blocks normed on both sides of their sublayers with gated, scaled results, windowed sigmoid
+    attention with pooled blocks, a state-space mixer, input-weighted experts, a looped stretch of layers
+    (models/layered.py)."""
+    model_type = "fizelix"
+
+
 MODEL_REGISTRY = {c.model_type: c for c in (GPT2LMHeadModel, GPTJForCausalLM, GPTBigCodeForCausalLM,
                                             LlamaForCausalLM, TimisunForCausalLM, BabotarForCausalLM,
-                                            LamisunForCausalLM)}
+                                            LamisunForCausalLM, FizelixForCausalLM)}

@@ -1162,3 +1162,235 @@ def lamisun_state_dict(cfg: ModelConfig, seed: int = 0) -> Dict[str, torch.Tenso
     """The random weights of :func:`random_lamisun_weights` under their checkpoint names (bf16; tests, examples)."""
     get = _lamisun_random(cfg, seed)
     return {n: get(n).to(torch.bfloat16) for n in lamisun_shapes(cfg)}
+
+
+# ------------------------------------------------------------------------------ sandwich-normed per-layer designs (Fizelix)
+@dataclass
+class PoolAttnWeights:
+    """Windowed sigmoid attention with pooled blocks: ``proj`` [q | k | v | sublayer gate rows padded to 8, W] (one
+    GEMM), ``cols`` the first row of each part (``rg``: the gate logits of the block's gated residual); ``pb`` fp32
+    [heads] the per-head score bias; ``freqs`` fp32 [rot.dims / 2] the pairs' angular steps per position (None: no
+    rotation), ``rot_key`` (dims, base): layers with the same rotation share a step's angles; ``o`` [W, heads * vdim]."""
+    proj: torch.Tensor
+    cols: Dict[str, int]
+    pb: torch.Tensor
+    freqs: Optional[torch.Tensor]
+    rot_key: Optional[tuple]
+    o: torch.Tensor
+
+    def tensors(self):
+        return [t for t in (self.proj, self.pb, self.freqs, self.o) if t is not None]
+
+
+@dataclass
+class SSDWeights:
+    """State-space mixer: ``proj`` [z | x | B | C | dt | sublayer gate rows padded to 8, W] (one GEMM), ``cols`` the
+    first row of z, xbc (x, B, C side by side: one convolution), dt and rg; ``conv`` [channels, taps] with bias
+    ``conv_b``; ``dt_bias``, ``A_log``, ``D`` fp32 [heads]; ``norm`` [heads * vdim]; ``o`` [W, heads * vdim]."""
+    proj: torch.Tensor
+    cols: Dict[str, int]
+    conv: torch.Tensor
+    conv_b: torch.Tensor
+    dt_bias: torch.Tensor
+    A_log: torch.Tensor
+    D: torch.Tensor
+    norm: torch.Tensor
+    o: torch.Tensor
+
+    def tensors(self):
+        return [self.proj, self.conv, self.conv_b, self.dt_bias, self.A_log, self.D, self.norm, self.o]
+
+
+@dataclass
+class SandwichBlockWeights:
+    """One block normed on both sides of its sublayers, x <- x + post * rms_norm(sigmoid(W_g h + b) * sublayer(h)), h =
+    rms_norm(x) * norm. All vectors fp32: ``norm1`` / ``norm2``; ``post1`` / ``post2`` = the output norm's weight times
+    the layer scale; ``rg1_b`` / ``rg2_b`` the gates' biases (the gates' matrices ride in the sublayers' first
+    GEMMs: ``mix.cols["rg"]``, ``rg2_col``). Token input: ``side_gate`` [d, W], ``side_proj`` [W, d] in the storage
+    type, ``side_norm`` fp32 [W], ``side_col`` the layer's first column in the token table."""
+    norm1: torch.Tensor
+    post1: torch.Tensor
+    rg1_b: torch.Tensor
+    mix: object
+    norm2: Optional[torch.Tensor] = None
+    post2: Optional[torch.Tensor] = None
+    rg2_b: Optional[torch.Tensor] = None
+    rg2_col: int = 0
+    mlp: Optional[object] = None
+    side_gate: Optional[torch.Tensor] = None
+    side_proj: Optional[torch.Tensor] = None
+    side_norm: Optional[torch.Tensor] = None
+    side_col: int = 0
+
+    def tensors(self):
+        out = [self.norm1, self.post1, self.rg1_b] + self.mix.tensors()
+        for t in (self.norm2, self.post2, self.rg2_b, self.side_gate, self.side_proj, self.side_norm):
+            if t is not None:
+                out.append(t)
+        if self.mlp is not None:
+            out += self.mlp.tensors()
+        return out
+
+
+def fizelix_shapes(cfg: ModelConfig) -> Dict[str, tuple]:
+    """Checkpoint tensor names of a Fizelix config and their shapes."""
+    W, L = cfg.hidden_size, len(cfg.layer_specs)
+    out = {"embed": (cfg.vocab_size, W), "final.norm": (W,), "head": (cfg.vocab_size, W)}
+    d = cfg.token_side_dim
+    if d:
+        out["side.embed"] = (cfg.vocab_size, L * d)
+    for i, spec in enumerate(cfg.layer_specs):
+        p, m = f"l{i}.", spec.mixer
+        for n in ("norm1", "norm1b", "ls1", "rg1.b"):
+            out[p + n] = (W,)
+        out[p + "rg1"] = (W, W)
+        if m.kind == "pool_attention":
+            out.update({p + "mix.q": (m.heads * m.dim, W), p + "mix.k": (m.kv_heads * m.dim, W),
+                        p + "mix.v": (m.kv_heads * m.vdim, W), p + "mix.pb": (m.heads,),
+                        p + "mix.o": (W, m.heads * m.vdim)})
+        else:
+            C = m.conv_channels
+            out.update({p + "mix.in": (2 * m.inner + 2 * m.groups * m.state + m.heads, W), p + "mix.conv": (C, m.conv),
+                        p + "mix.conv.b": (C,), p + "mix.dt_bias": (m.heads,), p + "mix.A_log": (m.heads,),
+                        p + "mix.D": (m.heads,), p + "mix.norm": (m.inner,), p + "mix.o": (W, m.inner)})
+        f = spec.mlp
+        if f is not None:
+            for n in ("norm2", "norm2b", "ls2", "rg2.b"):
+                out[p + n] = (W,)
+            out[p + "rg2"] = (W, W)
+            if f.kind == "dense":
+                out.update({p + "mlp.gate": (f.ff, W), p + "mlp.up": (f.ff, W), p + "mlp.down": (W, f.ff)})
+            else:
+                out[p + "mlp.router"] = (f.experts, W)
+                for k in range(f.experts):
+                    out.update({f"{p}mlp.e{k}.gate": (f.expert.ff, W), f"{p}mlp.e{k}.up": (f.expert.ff, W),
+                                f"{p}mlp.e{k}.down": (W, f.expert.ff)})
+                if f.shared is not None:
+                    out.update({p + "mlp.shared.gate": (f.shared.ff, W), p + "mlp.shared.up": (f.shared.ff, W),
+                                p + "mlp.shared.down": (W, f.shared.ff)})
+        if d:
+            out.update({p + "side.gate": (d, W), p + "side.proj": (W, d), p + "side.norm": (W,)})
+    return out
+
+
+def _fizelix_finish(cfg: ModelConfig, get, device, dtype) -> ModelWeights:
+    """``get(name)`` returns the checkpoint tensor of that name (CPU). Shapes are checked against the config. Every
+    sublayer's first GEMM also carries the matrix of the sublayer's output gate (attention: q | k | v | gate; state
+    space: in | gate; dense feed-forward: gate | up | gate of the residual; experts: beside the shared expert's
+    gate | up, or alone). Norm weights, layer scales and biases are kept in fp32; the output norm's weight and the
+    layer scale become one vector, the final norm's weight carries the logit scale."""
+    shapes = fizelix_shapes(cfg)
+
+    def g(name):
+        t = get(name)
+        if tuple(t.shape) != shapes[name]:
+            raise ValueError(f"{name} has shape {tuple(t.shape)}, the config says {shapes[name]}")
+        return t
+
+    def dev(t, dt=dtype):
+        return None if t is None else t.to(device=device, dtype=dt).contiguous()
+
+    def f32(t):
+        return dev(t.float(), torch.float32)
+    d = cfg.token_side_dim
+    layers = []
+    for i, spec in enumerate(cfg.layer_specs):
+        p, m = f"l{i}.", spec.mixer
+        if m.kind == "pool_attention":
+            proj, cols = _cat_rows([("q", g(p + "mix.q")), ("k", g(p + "mix.k")), ("v", g(p + "mix.v")),
+                                    ("rg", g(p + "rg1"))])
+            freqs = None
+            if m.rot is not None:
+                freqs = f32(torch.tensor([m.rot.base ** (-2.0 * j / m.rot.dims) for j in range(m.rot.dims // 2)],
+                                         dtype=torch.float64))
+            mix = PoolAttnWeights(dev(proj), cols, f32(g(p + "mix.pb")), freqs,
+                                  (m.rot.dims, m.rot.base) if m.rot is not None else None, dev(g(p + "mix.o")))
+        else:
+            proj, cols = _cat_rows([("z", g(p + "mix.in")), ("rg", g(p + "rg1"))])
+            cols["xbc"] = m.inner
+            cols["dt"] = 2 * m.inner + 2 * m.groups * m.state
+            mix = SSDWeights(dev(proj), cols, dev(g(p + "mix.conv")), dev(g(p + "mix.conv.b")),
+                             f32(g(p + "mix.dt_bias")), f32(g(p + "mix.A_log")), f32(g(p + "mix.D")),
+                             dev(g(p + "mix.norm")), dev(g(p + "mix.o")))
+        blk = SandwichBlockWeights(f32(g(p + "norm1")), f32(g(p + "norm1b").float() * g(p + "ls1").float()),
+                                   f32(g(p + "rg1.b")), mix)
+        f = spec.mlp
+        if f is not None:
+            blk.norm2, blk.rg2_b = f32(g(p + "norm2")), f32(g(p + "rg2.b"))
+            blk.post2 = f32(g(p + "norm2b").float() * g(p + "ls2").float())
+            if f.kind == "dense":
+                gu, cols = _cat_rows([("g", g(p + "mlp.gate")), ("u", g(p + "mlp.up")), ("rg", g(p + "rg2"))])
+                blk.mlp, blk.rg2_col = DenseMLPWeights(dev(gu), dev(g(p + "mlp.down"))), cols["rg"]
+            else:
+                E, q = f.experts, p + "mlp."
+                parts = [("rg", g(p + "rg2"))]
+                if f.shared is not None:
+                    parts = [("g", g(q + "shared.gate")), ("u", g(q + "shared.up"))] + parts
+                sgu, cols = _cat_rows(parts)
+                blk.mlp = MoEWeights(
+                    router=dev(g(q + "router")), correction=None,
+                    gate=dev(torch.stack([g(f"{q}e{k}.gate") for k in range(E)])),
+                    up=dev(torch.stack([g(f"{q}e{k}.up") for k in range(E)])),
+                    down=dev(torch.stack([g(f"{q}e{k}.down") for k in range(E)])),
+                    shared_gu=dev(sgu), shared_down=dev(g(q + "shared.down")) if f.shared is not None else None)
+                blk.rg2_col = cols["rg"]
+        if d:
+            blk.side_gate, blk.side_proj = dev(g(p + "side.gate")), dev(g(p + "side.proj"))
+            blk.side_norm, blk.side_col = f32(g(p + "side.norm")), i * d
+        layers.append(blk)
+    vp = math.ceil(cfg.vocab_size / 16) * 16
+    head = torch.zeros(vp, cfg.hidden_size, dtype=dtype, device=device)
+    head[:cfg.vocab_size].copy_(g("head").to(device=device, dtype=dtype))
+    extra = {"side": dev(g("side.embed"))} if d else {}
+    return ModelWeights(wte=dev(g("embed")), wpe=None, layers=layers,
+                        lnf_w=f32(g("final.norm").float() * cfg.logit_scale), lnf_b=None, head=Linear(head), extra=extra)
+
+
+def load_fizelix_weights(cfg: ModelConfig, reader, device="cpu", dtype=torch.bfloat16) -> ModelWeights:
+    return _fizelix_finish(cfg, lambda n: reader.get(n), device, dtype)
+
+
+def _fizelix_random(cfg: ModelConfig, seed: int, device="cpu"):
+    import zlib
+
+    shapes = fizelix_shapes(cfg)
+
+    def get(name: str) -> torch.Tensor:
+        gen = torch.Generator(device=device)
+        gen.manual_seed((seed * 1000003 + zlib.crc32(name.encode())) & 0x7FFFFFFF)
+        shp = shapes[name]
+        t = torch.randn(*shp, generator=gen, dtype=torch.float32, device=device)
+        last = name.split(".")[-1]
+        if name.endswith((".rg1.b", ".rg2.b", ".conv.b")):
+            t = 0.3 * t
+        elif last.startswith("norm") or name == "final.norm":
+            t = 1.0 + 0.1 * t
+        elif last in ("ls1", "ls2"):
+            t = 0.5 + 0.1 * t
+        elif last == "A_log":
+            t = 0.5 * t - 0.5
+        elif last in ("dt_bias", "pb"):
+            t = 0.5 * t - (1.0 if last == "pb" else 0.0)
+        elif last == "D":
+            t = 1.0 + 0.2 * t
+        elif last == "conv":
+            t = t * shp[1] ** -0.5
+        elif name == "embed":
+            t = t / max(cfg.embedding_scale, 1e-6)
+        elif len(shp) == 2 and name != "side.embed":
+            t = t * shp[1] ** -0.5
+        return t.to(torch.bfloat16).float()
+    return get
+
+
+def random_fizelix_weights(cfg: ModelConfig, device="cpu", dtype=torch.bfloat16, seed: int = 0) -> ModelWeights:
+    """Random-init weights of a Fizelix config (values rounded to bf16, so a bf16 and an fp32 run hold the same
+    model): projections ~ N(0, 1 / fan_in), norm weights around one, layer scales around one half."""
+    gen = device if torch.device(device).type == "cuda" else "cpu"  # large models: draw on the GPU
+    return _fizelix_finish(cfg, _fizelix_random(cfg, seed, gen), device, dtype)
+
+
+def fizelix_state_dict(cfg: ModelConfig, seed: int = 0) -> Dict[str, torch.Tensor]:
+    """The random weights of :func:`random_fizelix_weights` under their checkpoint names (bf16; tests, examples)."""
+    get = _fizelix_random(cfg, seed)
+    return {n: get(n).to(torch.bfloat16) for n in fizelix_shapes(cfg)}

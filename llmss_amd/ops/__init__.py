@@ -197,3 +197,11 @@ act_fn = _route("act_fn")
 rope_angles = _route("rope_angles")
 qk_norm_cache = _route("qk_norm_cache")
 diff_combine = _route("diff_combine")
+
+# ------------------- blocks normed on both sides / token input / windowed sigmoid attention with pooled blocks / SSD
+sandwich_add_norm = _route("sandwich_add_norm")
+token_side_add = _route("token_side_add")
+rope_pairs_cache = _route("rope_pairs_cache")
+pool_update = _route("pool_update")
+pool_window_attn = _route("pool_window_attn")
+ssd_recurrence = _route("ssd_recurrence")

@@ -574,30 +574,35 @@ def glu_clamp(gu: torch.Tensor, F_: int, limit: float, alpha: float) -> torch.Te
     return glu_clamped(gu[:, :F_].float(), gu[:, F_:2 * F_].float(), limit, alpha).to(gu.dtype)
 
 
-def moe_route(z: torch.Tensor, corr: Optional[torch.Tensor], top: int):
+def moe_route(z: torch.Tensor, corr: Optional[torch.Tensor], top: int, normalize: bool = True):
     """fp32 router logits [T, E] -> (idx int32 [T, top], weights fp32 [T, top]): scores sigmoid(z), the ``top``
-    largest of score + corr chosen (ties: lower index), weights = chosen scores / (their sum + 1e-20)."""
+    largest of score + corr chosen (ties: lower index), weights = chosen scores / (their sum + 1e-20), or the chosen
+    scores themselves (``normalize`` false)."""
     s = torch.sigmoid(z.float())
     ch = s if corr is None else s + corr.float()
     # descending by value, ascending by index among equals
     order = torch.argsort(ch, dim=-1, descending=True, stable=True)
     idx = order[:, :top]
     w = torch.gather(s, 1, idx)
-    w = w / (w.sum(-1, keepdim=True) + 1e-20)
+    if normalize:
+        w = w / (w.sum(-1, keepdim=True) + 1e-20)
     return idx.to(torch.int32), w
 
 
-def moe_router(h: torch.Tensor, router: torch.Tensor, corr: Optional[torch.Tensor], top: int):
+def moe_router(h: torch.Tensor, router: torch.Tensor, corr: Optional[torch.Tensor], top: int,
+               normalize: bool = True):
     """Router logits in fp32 from the layer input, then :func:`moe_route`."""
-    return moe_route(linear_f(h, router, torch.float32), corr, top)
+    return moe_route(linear_f(h, router, torch.float32), corr, top, normalize)
 
 
 def moe_experts(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate: torch.Tensor, up: torch.Tensor,
                 down: torch.Tensor, limit: float, alpha: float, shared: Optional[torch.Tensor] = None,
-                combine: bool = True) -> torch.Tensor:
+                combine: bool = True, act: str = "glu_clamp", weight_input: bool = False) -> torch.Tensor:
     """sum_j wts[t, j] * down_e(glu(gate_e h, up_e h)) (+ shared) with e = idx[t, j] -> fp32 [T, N]. Stacked expert
     weights gate / up [E, F, K], down [E, N, F]; the activation is rounded to the storage type between the
-    products, as the grouped GEMMs do."""
+    products, as the grouped GEMMs do. ``act`` "silu": silu(g) * u without clamps. ``weight_input``: the weight
+    multiplies the expert's input instead, sum_j down_e(act(w gate_e h, w up_e h)) (experts have no biases, so the
+    weight is applied to the two products)."""
     T = h.shape[0]
     N = down.shape[1]
     out = torch.zeros(T, N, dtype=torch.float32, device=h.device)
@@ -606,8 +611,11 @@ def moe_experts(h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, gate: tor
         for e in idx[:, j].unique().tolist():
             rows = torch.nonzero(idx[:, j] == e).flatten()
             x = hf[rows]
-            a = glu_clamped(x @ gate[e].float().t(), x @ up[e].float().t(), limit, alpha).to(h.dtype).float()
-            out[rows] += wts[rows, j:j + 1] * (a @ down[e].float().t())
+            g_, u_ = x @ gate[e].float().t(), x @ up[e].float().t()
+            if weight_input:
+                g_, u_ = g_ * wts[rows, j:j + 1], u_ * wts[rows, j:j + 1]
+            a = (g_ * torch.sigmoid(g_) * u_ if act == "silu" else glu_clamped(g_, u_, limit, alpha)).to(h.dtype).float()
+            out[rows] += (a @ down[e].float().t()) * (1.0 if weight_input else wts[rows, j:j + 1])
     if shared is not None:
         out += shared.float()
     return out
@@ -643,10 +651,11 @@ def stream_add_norm(x, y, mix, outw, c: float, inw, w, eps: float, rms: bool, ou
     return (u * torch.rsqrt(u.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
 
 
-def causal_conv(x, w, state, cu, ctx_lens, state_slots, residual: bool, silu: bool, out_dtype):
+def causal_conv(x, w, state, cu, ctx_lens, state_slots, residual: bool, silu: bool, out_dtype, bias=None):
     """Per-channel causal convolution over time of x [T, C] with w [C, taps] (last column: the current row), each
     sequence continuing from the taps - 1 inputs in its state slot (state fp32 [slots, taps - 1, C], renewed here;
-    a portion starting at position 0 reads zeros). ``residual`` adds x itself; ``silu`` applies x * sigmoid(x)."""
+    a portion starting at position 0 reads zeros). ``residual`` adds x itself; ``bias`` [C] is added to every row;
+    ``silu`` applies x * sigmoid(x)."""
     T, C = x.shape
     taps = w.shape[1]
     R = taps - 1
@@ -666,21 +675,30 @@ def causal_conv(x, w, state, cu, ctx_lens, state_slots, residual: bool, silu: bo
         y = sum(wf[:, k] * full[k:k + q] for k in range(taps))
         if residual:
             y = y + cur
+        if bias is not None:
+            y = y + bias.float()
         out[t0:t0 + q] = y
     if silu:
         out = out * torch.sigmoid(out)
     return out.to(out_dtype)
 
 
-def gated_group_norm(o, gate, w, eps: float, act: str, c: float, out=None, out_dtype=None):
+def gated_group_norm(o, gate, w, eps: float, act: str, c: float, out=None, out_dtype=None, groups: int = 0,
+                     gate_first: bool = False):
     """o fp32 [T, groups * n] divided per group of n = len(w) by its root mean square, times w, times act(gate)
-    (``sigmoid`` or ``silu``), times c; written to ``out`` (a [T, groups * n] view) when given."""
+    (``sigmoid`` or ``silu``), times c; written to ``out`` (a [T, groups * n] view) when given. ``groups`` > 0: w
+    holds a weight for every column ([groups * n]) instead of one per column of a group. ``gate_first``: the gate is
+    applied before the norm, rms_div(o * act(gate)) * w."""
     T, N = o.shape
-    n = w.numel()
-    og = o.float().view(T, N // n, n)
+    n = N // groups if groups else w.numel()
     g = gate.float()
     a = torch.sigmoid(g) if act == "sigmoid" else g * torch.sigmoid(g)
-    y = (og * torch.rsqrt(og.pow(2).mean(-1, keepdim=True) + eps) * w.float()).view(T, N) * a * c
+    of = o.float() * a if gate_first else o.float()
+    og = of.view(T, N // n, n)
+    y = og * torch.rsqrt(og.pow(2).mean(-1, keepdim=True) + eps)
+    y = (y.view(T, N) * w.float() if groups else (y * w.float()).view(T, N)) * c
+    if not gate_first:
+        y = y * a
     if out is not None:
         out.copy_(y)
         return out
@@ -947,3 +965,132 @@ def diff_combine(O, lam: float, eps: float, mult: float, heads: int, kv_heads: i
     o = Og[:, :, 0] - lam * Og[:, :, 1]
     o = o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * mult
     return o.reshape(T, heads * vdim).to(out_dtype)
+
+
+
+# ------------------- blocks normed on both sides / token input / windowed sigmoid attention with pooled blocks / SSD
+def sandwich_add_norm(x, y, r, rb, wpost, eps: float, add, wnext, out_dtype):
+    """x fp32 [T, W], in place: with ``y`` [T, W], x += rms_norm(y * sigmoid(r + rb)) * wpost (``r`` [T, W] gate
+    logits and ``rb`` [W] their bias, or None for no gate; ``wpost`` fp32 [W]); with ``add`` (fp32 [T, W]) x += add;
+    with ``wnext`` (fp32 [W]) returns rms_norm(x) * wnext in ``out_dtype``, else None."""
+    if y is not None:
+        yf = y.float()
+        if r is not None:
+            yf = yf * torch.sigmoid(r.float() + rb.float())
+        x.add_(yf * torch.rsqrt(yf.pow(2).mean(-1, keepdim=True) + eps) * wpost.float())
+    if add is not None:
+        x.add_(add)
+    if wnext is None:
+        return None
+    return (x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * wnext.float()).to(out_dtype)
+
+
+def token_side_add(x, ids, table, col0: int, gate_w, proj_w, norm_w, eps: float, add, wnext, out_dtype):
+    """x fp32 [T, W], in place: e = table[ids, col0 : col0 + d] (d = rows of gate_w); g = gelu_tanh(gate_w x) * e;
+    y = proj_w g; x += rms_norm(y) * norm_w. Then ``add`` and ``wnext`` as in :func:`sandwich_add_norm`."""
+    d = gate_w.shape[0]
+    e = table[ids.clamp(0, table.shape[0] - 1), col0:col0 + d].float()
+    g = torch.nn.functional.gelu(x @ gate_w.float().t(), approximate="tanh") * e
+    y = g @ proj_w.float().t()
+    x.add_(y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float())
+    return sandwich_add_norm(x, None, None, None, None, eps, add, wnext, out_dtype)
+
+
+def rope_pairs_cache(proj, off_q: int, off_k: int, off_v: int, cs, k_cache, v_cache, slots, heads: int,
+                     kv_heads: int, dim: int, vdim: int):
+    """From the projection rows: q and k with the neighbouring pairs (2i, 2i + 1), i < cs.shape[1], of every head
+    turned by ``cs`` [T, dims / 2, 2] = (cos, sin) (None: no rotation), v as it is. Returns q fp32 [T, heads * dim];
+    k / v go into the paged caches [blocks, block_size, kv_heads * dim | kv_heads * vdim] at ``slots`` (< 0: not
+    cached)."""
+    T = proj.shape[0]
+    nq, nk, nv = heads * dim, kv_heads * dim, kv_heads * vdim
+    q = proj[:, off_q:off_q + nq].float().reshape(T, heads, dim)
+    k = proj[:, off_k:off_k + nk].float().reshape(T, kv_heads, dim)
+    if cs is not None:
+        q, k = _turn_neighbours(q, cs), _turn_neighbours(k, cs)
+    keep = slots >= 0
+    k_cache.view(-1, nk)[slots[keep]] = k.reshape(T, nk)[keep].to(k_cache.dtype)
+    v_cache.view(-1, nv)[slots[keep]] = proj[:, off_v:off_v + nv][keep].to(v_cache.dtype)
+    return q.reshape(T, nq).contiguous()
+
+
+def pool_slot(block_tables, b: int, blk: int, pool: int, bs: int, per: int):
+    """Row of the pooled caches that holds block ``blk`` of sequence ``b``: the page of the block's first position,
+    and within it the block's rank among the blocks that start there."""
+    p = blk * pool
+    return int(block_tables[b, p // bs]) * per + (p % bs) // pool
+
+
+def pool_update(k_cache, v_cache, kp_cache, vp_cache, block_tables, cu, ctx_lens, pool: int):
+    """Mean key and mean value (fp32) of every block of ``pool`` positions whose last position the step has just
+    written, from the cached rows of the block: kp_cache / vp_cache fp32 [blocks, ceil(block_size / pool), kv_heads *
+    dim | vdim], row :func:`pool_slot`."""
+    bs, per = k_cache.shape[1], kp_cache.shape[1]
+    nk, nv = k_cache.shape[2], v_cache.shape[2]
+    for b, _, n, p0 in _seq_rows(cu, ctx_lens):
+        L = p0 + n
+        for blk in range(p0 // pool, L // pool):  # p0 <= blk * pool + pool - 1 < L
+            pos = torch.arange(blk * pool, blk * pool + pool)
+            rows = block_tables[b, pos // bs].long() * bs + pos % bs
+            s = pool_slot(block_tables, b, blk, pool, bs, per)
+            kp_cache.view(-1, nk)[s] = k_cache.view(-1, nk)[rows].float().mean(0)
+            vp_cache.view(-1, nv)[s] = v_cache.view(-1, nv)[rows].float().mean(0)
+
+
+def pool_window_attn(q, k_cache, v_cache, kp_cache, vp_cache, block_tables, cu, ctx_lens, pb, heads: int,
+                     kv_heads: int, dim: int, vdim: int, scale: float, window: int, pool: int, out_dtype,
+                     max_qlen: int = 0, num_decode: int = 0):
+    """Sigmoid-weighted attention of every row over its sequence's cache: the row at position i adds sigmoid(q . k *
+    scale + pb[head]) * v over the positions j with 0 <= i - j (< window when window > 0) and, when ``pool`` > 0, over
+    the pooled rows of the blocks with blk * pool + pool - 1 <= i - window. q fp32 [T, heads * dim]; returns [T, heads
+    * vdim] in ``out_dtype``. ``max_qlen`` and ``num_decode`` only steer the GPU kernels."""
+    T = q.shape[0]
+    bs = k_cache.shape[1]
+    rep = heads // kv_heads
+    out = torch.zeros(T, heads, vdim, dtype=torch.float32)
+    per = kp_cache.shape[1] if pool else 0
+    for b, t0, n, p0 in _seq_rows(cu, ctx_lens):
+        L = p0 + n
+        blocks = block_tables[b, : -(-L // bs)].long()
+        K = k_cache[blocks].reshape(-1, kv_heads, dim)[:L].float()
+        V = v_cache[blocks].reshape(-1, kv_heads, vdim)[:L].float()
+        nb = max(0, (L - window) // pool) if pool and window else 0
+        if nb:
+            rows = torch.tensor([pool_slot(block_tables, b, j, pool, bs, per) for j in range(nb)])
+            K = torch.cat([K, kp_cache.view(-1, kv_heads, dim)[rows].float()], 0)
+            V = torch.cat([V, vp_cache.view(-1, kv_heads, vdim)[rows].float()], 0)
+        qq = q[t0:t0 + n].view(n, heads, dim).float()
+        s = torch.einsum("nhd,lhd->hnl", qq, K.repeat_interleave(rep, 1)) * scale + pb.float()[:, None, None]
+        i = (p0 + torch.arange(n))[:, None]
+        j = torch.arange(L)[None, :]
+        vis = (j <= i) & ((i - j < window) if window else torch.ones_like(j <= i))
+        if nb:
+            last = (torch.arange(nb) * pool + pool - 1)[None, :]
+            vis = torch.cat([vis, last <= i - window], 1)
+        p = torch.sigmoid(s) * vis
+        out[t0:t0 + n] = torch.einsum("hnl,lhv->nhv", p, V.repeat_interleave(rep, 1))
+    return out.reshape(T, heads * vdim).to(out_dtype)
+
+
+def ssd_recurrence(x, Bm, Cm, dt, A_log, dt_bias, D, state, cu, ctx_lens, state_slots, heads: int, groups: int,
+                   N: int, vdim: int):
+    """Per head h (group g = h // (heads / groups)) over each sequence's rows: d = softplus(dt + dt_bias_h);
+    S <- exp(-exp(A_log_h) d) S + d B_g x_h^T; y = S^T C_g + D_h x_h, S fp32 [slots, heads, N, vdim] carried in the
+    sequence's slot (zero when the portion starts at position 0). x [T, heads * vdim], Bm / Cm [T, groups * N], dt [T,
+    heads]. Returns fp32 [T, heads * vdim]."""
+    T = x.shape[0]
+    rep = heads // groups
+    out = torch.zeros(T, heads * vdim, dtype=torch.float32)
+    slots = state_slots.tolist()
+    for b, t0, n, p0 in _seq_rows(cu, ctx_lens):
+        S = state[slots[b]].clone() if p0 > 0 else torch.zeros(heads, N, vdim)
+        xx = x[t0:t0 + n].float().view(n, heads, vdim)
+        BB = Bm[t0:t0 + n].float().view(n, groups, N).repeat_interleave(rep, 1)
+        CC = Cm[t0:t0 + n].float().view(n, groups, N).repeat_interleave(rep, 1)
+        d = torch.nn.functional.softplus(dt[t0:t0 + n].float() + dt_bias.float(), threshold=20.0)
+        a = torch.exp(-torch.exp(A_log.float()) * d)
+        for j in range(n):
+            S = a[j][:, None, None] * S + (d[j][:, None] * BB[j])[:, :, None] * xx[j][:, None, :]
+            out[t0 + j] = (torch.einsum("hdv,hd->hv", S, CC[j]) + D.float()[:, None] * xx[j]).reshape(-1)
+        state[slots[b]] = S
+    return out
