@@ -87,7 +87,7 @@ void launch_gemm_tile(const void* A, const void* B, void* C, int M, int N, int K
                       int64_t sBb, int64_t sBn, int64_t sCb, int64_t sCm, int dc, hipStream_t st);
 void launch_moe_gate_up_tile(const void* h, int64_t ldh, const void* wg, const void* wu, const void* meta,
                              const void* order, void* act, int E, int maxt, int top, int F, int K, float limit,
-                             float alpha, int tile_rows, hipStream_t st);
+                             float alpha, int tile_rows, const void* pw, int silu, hipStream_t st);
 void launch_moe_down_tile(const void* act, const void* wd, const void* meta, void* y, int E, int maxt, int N, int F,
                           int tile_rows, hipStream_t st);
 void launch_latent_norm_cache(const void* src, int64_t ld, int off, const void* w, float eps, void* cache,
@@ -97,14 +97,15 @@ void launch_rope_angles(const void* positions, const void* freqs, void* cs, int 
 void launch_latent_attn(const void* qa, int64_t ldq, const void* cache, const void* bt, int maxb, const void* cu_q,
                         const void* ctx_lens, void* out, int64_t ldo, int T_, int B, int H, int R, int bs, int window,
                         float scale, int dt, hipStream_t st);
-void launch_moe_route(const void* z, const void* corr, void* idx, void* wts, int T_, int E, int top, hipStream_t st);
+void launch_moe_route(const void* z, const void* corr, void* idx, void* wts, int T_, int E, int top, int norm,
+                      hipStream_t st);
 void launch_moe_router(const void* h, int64_t ldh, const void* wr, const void* corr, void* idx, void* wts, int T_,
-                       int E, int K, int top, int dt, hipStream_t st);
+                       int E, int K, int top, int dt, int norm, hipStream_t st);
 void launch_moe_group(const void* idx, int P, int E, int maxt, void* meta, void* order, void* place, int tile_rows,
                       hipStream_t st);
 void launch_moe_gate_up(const void* h, int64_t ldh, const void* wg, const void* wu, const void* meta,
                         const void* order, void* act, int E, int maxt, int top, int F, int K, float limit,
-                        float alpha, int dt, hipStream_t st);
+                        float alpha, int dt, const void* pw, int silu, hipStream_t st);
 void launch_moe_down(const void* act, const void* wd, const void* meta, void* y, int E, int maxt, int N, int F,
                      int dt, hipStream_t st);
 void launch_moe_combine(const void* y, const void* place, const void* wts, const void* shared_, int64_t lds_,
@@ -120,16 +121,35 @@ void launch_stream_add_norm(void* x, const void* y, int64_t ldy, const void* mix
                             int W, int dt, int h_f32, hipStream_t st);
 void launch_causal_conv(const void* in, int64_t ldi, const void* w, void* state, const void* cu, const void* ctx,
                         const void* sslots, void* out, int64_t ldo, int T_, int B, int C, int taps, int res, int silu,
-                        int di, int dw, int dout, hipStream_t st);
+                        int di, int dw, int dout, const void* bias, hipStream_t st);
 void launch_gated_group_norm(const void* o, int64_t ldo, const void* gate, int64_t ldg, const void* w, float eps,
-                             int act, float c, void* out, int64_t ldout, int T_, int groups, int n, int dt,
-                             hipStream_t st);
+                             int act, float c, void* out, int64_t ldout, int T_, int groups, int n, int dt, int wfull,
+                             int first, hipStream_t st);
 void launch_glu_act(const void* gu, int64_t ldg, void* out, int64_t ldo, int T_, int F, int act, int dt,
                     hipStream_t st);
 void launch_recurrence(int mode, const void* q, const void* k, const void* v, int64_t ldq, int64_t ldk, int64_t ldv,
                        const void* ab, int64_t ldab, int off_a, int off_b, const void* decay, const void* dt_bias,
                        void* state, const void* cu, const void* ctx, const void* sslots, void* out, int64_t ldo, int B,
-                       int H, int G, int dim, int vdim, int silu_in, int gates_ready, int dq, int dp, hipStream_t st);
+                       int H, int G, int dim, int vdim, int silu_in, int gates_ready, int dq, int dp, const void* skip,
+                       hipStream_t st);
+// blocks normed on both sides, token input, windowed sigmoid attention with pooled blocks
+void launch_sandwich_add_norm(void* x, const void* y, int64_t ldy, const void* ey, const void* place, const void* wts,
+                              int top, const void* shared_, int64_t lds_, const void* r, int64_t ldr, const void* rb,
+                              const void* wpost, const void* add, const void* wnext, void* h, int64_t ldh, float eps,
+                              int T_, int W, int dt, hipStream_t st);
+void launch_token_side_add(void* x, const void* ids, const void* table, int64_t ldt, int vocab, int col0, int d,
+                           const void* wg, const void* wp, const void* wn, const void* add, const void* wnext, void* h,
+                           int64_t ldh, float eps, int T_, int W, int dt, hipStream_t st);
+void launch_rope_pairs_cache(const void* proj, int64_t ldp, int off_q, int off_k, int off_v, const void* cs, int rdims,
+                             void* qout, void* kc, void* vc, const void* slots, int T_, int H, int G, int dim, int vdim,
+                             int dt, hipStream_t st);
+void launch_pool_update(const void* kc, const void* vc, void* kp, void* vp, const void* bt, int maxb, const void* cu,
+                        const void* ctx, int B, int max_qlen, int nk, int nv, int bs, int pool, int per, int dt,
+                        hipStream_t st);
+void launch_pool_window_attn(const void* q, const void* kc, const void* vc, const void* kp, const void* vp,
+                             const void* bt, int maxb, const void* cu, const void* ctx, const void* pb, void* out,
+                             int out_f32, int T_, int B, int H, int G, int dim, int vdim, int bs, float scale,
+                             int window, int pool, int per, int dt, hipStream_t st);
 void launch_silu_f32(const void* in, int64_t ldi, void* out, int64_t ldo, int T_, int n, int dt, hipStream_t st);
 void launch_delta_gates(const void* a, const void* b, int64_t ld, const void* A_log, const void* dt_bias, void* gates,
                         int T_, int H, int dt, hipStream_t st);
@@ -319,9 +339,9 @@ PYBIND11_MODULE(_C, m) {
   });
   m.def("moe_gate_up_tile", [](uintptr_t h, int64_t ldh, uintptr_t wg, uintptr_t wu, uintptr_t meta, uintptr_t order,
                                uintptr_t act, int E, int maxt, int top, int F, int K, float limit, float alpha,
-                               int tile_rows, uintptr_t st) {
+                               int tile_rows, uintptr_t pw, int silu, uintptr_t st) {
     launch_moe_gate_up_tile(CP(h), ldh, CP(wg), CP(wu), CP(meta), CP(order), P(act), E, maxt, top, F, K, limit, alpha,
-                            tile_rows, S(st));
+                            tile_rows, CP(pw), silu, S(st));
   });
   m.def("moe_down_tile", [](uintptr_t act, uintptr_t wd, uintptr_t meta, uintptr_t y, int E, int maxt, int N, int F,
                             int tile_rows, uintptr_t st) {
@@ -342,11 +362,11 @@ PYBIND11_MODULE(_C, m) {
     launch_latent_attn(CP(qa), ldq, CP(cache), CP(bt), maxb, CP(cu), CP(ctx), P(out), ldo, T, B, H, R, bs, window,
                        scale, dt, S(st));
   });
-  m.def("moe_route", [](uintptr_t z, uintptr_t corr, uintptr_t idx, uintptr_t wts, int T, int E, int top,
-                        uintptr_t st) { launch_moe_route(CP(z), CP(corr), P(idx), P(wts), T, E, top, S(st)); });
+  m.def("moe_route", [](uintptr_t z, uintptr_t corr, uintptr_t idx, uintptr_t wts, int T, int E, int top, int norm,
+                        uintptr_t st) { launch_moe_route(CP(z), CP(corr), P(idx), P(wts), T, E, top, norm, S(st)); });
   m.def("moe_router", [](uintptr_t h, int64_t ldh, uintptr_t wr, uintptr_t corr, uintptr_t idx, uintptr_t wts, int T,
-                         int E, int K, int top, int dt, uintptr_t st) {
-    launch_moe_router(CP(h), ldh, CP(wr), CP(corr), P(idx), P(wts), T, E, K, top, dt, S(st));
+                         int E, int K, int top, int dt, int norm, uintptr_t st) {
+    launch_moe_router(CP(h), ldh, CP(wr), CP(corr), P(idx), P(wts), T, E, K, top, dt, norm, S(st));
   });
   m.def("moe_group", [](uintptr_t idx, int Pn, int E, int maxt, uintptr_t meta, uintptr_t order, uintptr_t place,
                         int tile_rows, uintptr_t st) {
@@ -354,9 +374,9 @@ PYBIND11_MODULE(_C, m) {
   });
   m.def("moe_gate_up", [](uintptr_t h, int64_t ldh, uintptr_t wg, uintptr_t wu, uintptr_t meta, uintptr_t order,
                           uintptr_t act, int E, int maxt, int top, int F, int K, float limit, float alpha, int dt,
-                          uintptr_t st) {
+                          uintptr_t pw, int silu, uintptr_t st) {
     launch_moe_gate_up(CP(h), ldh, CP(wg), CP(wu), CP(meta), CP(order), P(act), E, maxt, top, F, K, limit, alpha, dt,
-                       S(st));
+                       CP(pw), silu, S(st));
   });
   m.def("moe_down", [](uintptr_t act, uintptr_t wd, uintptr_t meta, uintptr_t y, int E, int maxt, int N, int F, int dt,
                        uintptr_t st) { launch_moe_down(CP(act), CP(wd), CP(meta), P(y), E, maxt, N, F, dt, S(st)); });
@@ -378,22 +398,26 @@ PYBIND11_MODULE(_C, m) {
   });
   m.def("causal_conv", [](uintptr_t in, int64_t ldi, uintptr_t w, uintptr_t state, uintptr_t cu, uintptr_t ctx,
                           uintptr_t ss, uintptr_t out, int64_t ldo, int T, int B, int C, int taps, int res, int silu,
-                          int di, int dw, int dout, uintptr_t st) {
+                          int di, int dw, int dout, uintptr_t bias, uintptr_t st) {
     launch_causal_conv(CP(in), ldi, CP(w), P(state), CP(cu), CP(ctx), CP(ss), P(out), ldo, T, B, C, taps, res, silu,
-                       di, dw, dout, S(st));
+                       di, dw, dout, CP(bias), S(st));
   });
   m.def("gated_group_norm", [](uintptr_t o, int64_t ldo, uintptr_t gate, int64_t ldg, uintptr_t w, float eps, int act,
-                               float c, uintptr_t out, int64_t ldout, int T, int groups, int n, int dt, uintptr_t st) {
-    launch_gated_group_norm(CP(o), ldo, CP(gate), ldg, CP(w), eps, act, c, P(out), ldout, T, groups, n, dt, S(st));
+                               float c, uintptr_t out, int64_t ldout, int T, int groups, int n, int dt, int wfull,
+                               int first, uintptr_t st) {
+    launch_gated_group_norm(CP(o), ldo, CP(gate), ldg, CP(w), eps, act, c, P(out), ldout, T, groups, n, dt, wfull,
+                            first, S(st));
   });
   m.def("glu_act", [](uintptr_t gu, int64_t ldg, uintptr_t out, int64_t ldo, int T, int F, int act, int dt,
                       uintptr_t st) { launch_glu_act(CP(gu), ldg, P(out), ldo, T, F, act, dt, S(st)); });
   m.def("recurrence", [](int mode, uintptr_t q, uintptr_t k, uintptr_t v, int64_t ldq, int64_t ldk, int64_t ldv,
                          uintptr_t ab, int64_t ldab, int off_a, int off_b, uintptr_t decay, uintptr_t dtb,
                          uintptr_t state, uintptr_t cu, uintptr_t ctx, uintptr_t ss, uintptr_t out, int64_t ldo, int B,
-                         int H, int G, int dim, int vdim, int silu_in, int gates_ready, int dq, int dp, uintptr_t st) {
+                         int H, int G, int dim, int vdim, int silu_in, int gates_ready, int dq, int dp, uintptr_t skip,
+                         uintptr_t st) {
     launch_recurrence(mode, CP(q), CP(k), CP(v), ldq, ldk, ldv, CP(ab), ldab, off_a, off_b, CP(decay), CP(dtb),
-                      P(state), CP(cu), CP(ctx), CP(ss), P(out), ldo, B, H, G, dim, vdim, silu_in, gates_ready, dq, dp, S(st));
+                      P(state), CP(cu), CP(ctx), CP(ss), P(out), ldo, B, H, G, dim, vdim, silu_in, gates_ready, dq, dp,
+                      CP(skip), S(st));
   });
   m.def("silu_f32", [](uintptr_t in, int64_t ldi, uintptr_t out, int64_t ldo, int T, int n, int dt, uintptr_t st) {
     launch_silu_f32(CP(in), ldi, P(out), ldo, T, n, dt, S(st));
@@ -450,6 +474,38 @@ PYBIND11_MODULE(_C, m) {
   m.def("diff_combine", [](uintptr_t O, float lam, float eps, float mult, uintptr_t y, int64_t ldy, int T, int H, int G,
                            int vdim, int dt, uintptr_t st) {
     launch_diff_combine(CP(O), lam, eps, mult, P(y), ldy, T, H, G, vdim, dt, S(st));
+  });
+  m.def("sandwich_add_norm", [](uintptr_t x, uintptr_t y, int64_t ldy, uintptr_t ey, uintptr_t place, uintptr_t wts,
+                                int top, uintptr_t sh, int64_t lds_, uintptr_t r, int64_t ldr, uintptr_t rb,
+                                uintptr_t wpost, uintptr_t add, uintptr_t wnext, uintptr_t h, int64_t ldh, float eps,
+                                int T, int W, int dt, uintptr_t st) {
+    launch_sandwich_add_norm(P(x), CP(y), ldy, CP(ey), CP(place), CP(wts), top, CP(sh), lds_, CP(r), ldr, CP(rb),
+                             CP(wpost), CP(add), CP(wnext), P(h), ldh, eps, T, W, dt, S(st));
+  });
+  m.def("token_side_add", [](uintptr_t x, uintptr_t ids, uintptr_t table, int64_t ldt, int vocab, int col0, int d,
+                             uintptr_t wg, uintptr_t wp, uintptr_t wn, uintptr_t add, uintptr_t wnext, uintptr_t h,
+                             int64_t ldh, float eps, int T, int W, int dt, uintptr_t st) {
+    launch_token_side_add(P(x), CP(ids), CP(table), ldt, vocab, col0, d, CP(wg), CP(wp), CP(wn), CP(add), CP(wnext),
+                          P(h), ldh, eps, T, W, dt, S(st));
+  });
+  m.def("rope_pairs_cache", [](uintptr_t proj, int64_t ldp, int off_q, int off_k, int off_v, uintptr_t cs, int rdims,
+                               uintptr_t qout, uintptr_t kc, uintptr_t vc, uintptr_t slots, int T, int H, int G,
+                               int dim, int vdim, int dt, uintptr_t st) {
+    launch_rope_pairs_cache(CP(proj), ldp, off_q, off_k, off_v, CP(cs), rdims, P(qout), P(kc), P(vc), CP(slots), T, H,
+                            G, dim, vdim, dt, S(st));
+  });
+  m.def("pool_update", [](uintptr_t kc, uintptr_t vc, uintptr_t kp, uintptr_t vp, uintptr_t bt, int maxb, uintptr_t cu,
+                          uintptr_t ctx, int B, int max_qlen, int nk, int nv, int bs, int pool, int per, int dt,
+                          uintptr_t st) {
+    launch_pool_update(CP(kc), CP(vc), P(kp), P(vp), CP(bt), maxb, CP(cu), CP(ctx), B, max_qlen, nk, nv, bs, pool, per,
+                       dt, S(st));
+  });
+  m.def("pool_window_attn", [](uintptr_t q, uintptr_t kc, uintptr_t vc, uintptr_t kp, uintptr_t vp, uintptr_t bt,
+                               int maxb, uintptr_t cu, uintptr_t ctx, uintptr_t pb, uintptr_t out, int out_f32, int T,
+                               int B, int H, int G, int dim, int vdim, int bs, float scale, int window, int pool,
+                               int per, int dt, uintptr_t st) {
+    launch_pool_window_attn(CP(q), CP(kc), CP(vc), CP(kp), CP(vp), CP(bt), maxb, CP(cu), CP(ctx), CP(pb), P(out),
+                            out_f32, T, B, H, G, dim, vdim, bs, scale, window, pool, per, dt, S(st));
   });
   register_runtime(m);
   register_comm(m);

@@ -31,9 +31,12 @@ struct GemmTileArgs {
   const int* order;
   int E, maxt, top;
   float limit, alpha;
+  const float* pw;  // GATE_UP: weight of each (token, slot) pair on the expert's input (null: 1)
+  int silu;         // GATE_UP: silu(g) * u instead of the clamped form
 };
 
-__device__ __forceinline__ float glu_clamped_t(float g, float u, float limit, float alpha) {
+__device__ __forceinline__ float glu_clamped_t(float g, float u, float limit, float alpha, int silu) {
+  if (silu) return g / (1.f + expf(-g)) * u;
   g = fminf(g, limit);
   u = fminf(fmaxf(u, -limit), limit);
   return g / (1.f + expf(-alpha * g)) * (u + 1.f);
@@ -178,12 +181,14 @@ __global__ __launch_bounds__(256) void gemm_tile_kernel(GemmTileArgs p) {
       const int r = wm + 16 * i + 4 * g + q;
       if (r >= rows) continue;
       TC* crow = C + (int64_t)((MODE == GT_PLAIN ? m0 : crow0) + r) * p.sCm;
+      float sw = 1.0f;
+      if constexpr (MODE == GT_GATE_UP) sw = p.pw ? p.pw[p.order[crow0 + r]] : 1.0f;
 #pragma unroll
       for (int j = 0; j < NB; ++j) {
         const int n = n0 + wn + 16 * j + li;
         if (n >= p.N) continue;
         float v = acc[i][j][q];
-        if constexpr (DUAL) v = glu_clamped_t(v, acc2[i][j][q], p.limit, p.alpha);
+        if constexpr (DUAL) v = glu_clamped_t(v * sw, acc2[i][j][q] * sw, p.limit, p.alpha, p.silu);
         El<TC>::st(crow + n, v);
       }
     }
@@ -214,7 +219,7 @@ void launch_gemm_tile(const void* A, const void* B, void* C, int M, int N, int K
 // per tile the list was built with (moe_group): 64 or 128
 void launch_moe_gate_up_tile(const void* h, int64_t ldh, const void* wg, const void* wu, const void* meta,
                              const void* order, void* act, int E, int maxt, int top, int F, int K, float limit,
-                             float alpha, int tile_rows, hipStream_t st) {
+                             float alpha, int tile_rows, const void* pw, int silu, hipStream_t st) {
   if (tile_rows != 64 && tile_rows != 128) throw std::runtime_error("moe_gate_up: tile rows must be 64 or 128");
   if (maxt <= 0) return;
   if (maxt > 65535) throw std::runtime_error("moe_gate_up: too many row tiles");
@@ -222,7 +227,7 @@ void launch_moe_gate_up_tile(const void* h, int64_t ldh, const void* wg, const v
   a.A = (const bf16_t*)h; a.B = (const bf16_t*)wg; a.B2 = (const bf16_t*)wu; a.C = act;
   a.N = F; a.K = K; a.sAm = ldh; a.sBb = (int64_t)F * K; a.sBn = K; a.sCm = F;
   a.meta = (const int*)meta; a.order = (const int*)order; a.E = E; a.maxt = maxt; a.top = top;
-  a.limit = limit; a.alpha = alpha;
+  a.limit = limit; a.alpha = alpha; a.pw = (const float*)pw; a.silu = silu;
   // 128-row tiles are 64 columns wide here: with two accumulator sets (gate and up) a 128x128 tile leaves one
   // workgroup per CU; at 128x64 two to three fit and hide each other's staging
   dim3 g((F + 63) / 64, maxt);

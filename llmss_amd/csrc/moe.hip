@@ -8,7 +8,8 @@
 //                grouped GEMMs launch a grid whose size is known on the host (ceil(P / rows) + E tiles at most)
 //   moe_gate_up: act[r, f] = glu(h[token(r)] . gate_e[f], h[token(r)] . up_e[f])   for sorted row r of expert e
 //   moe_down:    y[r, n] = act[r, :] . down_e[n, :]                   (fp32)
-//   moe_combine: out[t, :] = sum_j wts[t, j] * y[place[t * top + j], :] (+ shared[t, :])   (fp32, j ascending)
+//   moe_combine: out[t, :] = sum_j wts[t, j] * y[place[t * top + j], :] (+ shared[t, :])   (fp32, j ascending;
+//                no wts: the plain sum, for layers whose weights went onto the experts' inputs in moe_gate_up)
 //
 // Expert activation (clamped, gated): g = min(g, limit), u = clamp(u, -limit, limit),
 // glu = g * sigmoid(alpha * g) * (u + 1). glu_clamp applies the same to a dense [T, 2F] gate|up product (the
@@ -25,11 +26,16 @@ __device__ __forceinline__ float glu_clamped(float g, float u, float limit, floa
   u = fminf(fmaxf(u, -limit), limit);
   return g / (1.f + expf(-alpha * g)) * (u + 1.f);
 }
+// silu: the plain gated form silu(g) * u, no clamps
+__device__ __forceinline__ float glu_value(float g, float u, float limit, float alpha, int silu) {
+  return silu ? g / (1.f + expf(-g)) * u : glu_clamped(g, u, limit, alpha);
+}
 
 // ------------------------------------------------------------------------------------------------ routing
 // one wave per token; lanes over experts
 __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__ z, const float* __restrict__ corr,
-                                                       int* __restrict__ idx, float* __restrict__ wts, int E, int top) {
+                                                       int* __restrict__ idx, float* __restrict__ wts, int E, int top,
+                                                       int norm) {
   extern __shared__ float sc[];  // [E] scores, [E] choice values
   float* ch = sc + E;
   const int t = blockIdx.x, lane = threadIdx.x;
@@ -69,15 +75,17 @@ __global__ __launch_bounds__(64) void moe_route_kernel(const float* __restrict__
     }
     __syncthreads();
   }
+  if (!norm) return;  // the chosen scores themselves
   const float inv = 1.f / (sum + 1e-20f);
   for (int j = lane; j < top; j += 64) wts[(int64_t)t * top + j] *= inv;
 }
 
-void launch_moe_route(const void* z, const void* corr, void* idx, void* wts, int T_, int E, int top, hipStream_t st) {
+void launch_moe_route(const void* z, const void* corr, void* idx, void* wts, int T_, int E, int top, int norm,
+                      hipStream_t st) {
   if (T_ == 0) return;
   if (top > E || top <= 0) throw std::runtime_error("moe_route: top must be in [1, experts]");
   moe_route_kernel<<<T_, 64, 2 * E * sizeof(float), st>>>((const float*)z, (const float*)corr, (int*)idx, (float*)wts,
-                                                           E, top);
+                                                           E, top, norm);
   HIP_CHECK_LAUNCH();
 }
 
@@ -87,7 +95,8 @@ void launch_moe_route(const void* z, const void* corr, void* idx, void* wts, int
 template <typename T>
 __global__ __launch_bounds__(1024) void moe_router_kernel(const T* __restrict__ h, int64_t ldh, const T* __restrict__ wr,
                                                          const float* __restrict__ corr, int* __restrict__ idx,
-                                                         float* __restrict__ wts, int E, int K, int top, bool vec) {
+                                                         float* __restrict__ wts, int E, int K, int top, bool vec,
+                                                         int norm) {
   extern __shared__ float sc[];  // [E] scores, [E] choice values
   float* ch = sc + E;
   const int t = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wv = tid >> 6, nw = blockDim.x >> 6;
@@ -142,19 +151,21 @@ __global__ __launch_bounds__(1024) void moe_router_kernel(const T* __restrict__ 
     }
     __syncthreads();
   }
+  if (!norm) return;
   const float inv = 1.f / (sum + 1e-20f);
   for (int j = tid; j < top; j += blockDim.x) wts[(int64_t)t * top + j] *= inv;
 }
 
 void launch_moe_router(const void* h, int64_t ldh, const void* wr, const void* corr, void* idx, void* wts, int T_,
-                       int E, int K, int top, int dt, hipStream_t st) {
+                       int E, int K, int top, int dt, int norm, hipStream_t st) {
   if (T_ == 0) return;
   if (top > E || top <= 0) throw std::runtime_error("moe_router: top must be in [1, experts]");
   const int es = dt == 0 ? 2 : 4;
   const bool vec = K % 8 == 0 && ((uintptr_t)h % 16) == 0 && ((uintptr_t)wr % 16) == 0 && (ldh * es) % 16 == 0;
   const int threads = E >= 16 ? 1024 : (E >= 8 ? 512 : 256);  // a wave per expert up to 16 waves
   DISPATCH_T(dt, T, (moe_router_kernel<T><<<T_, threads, 2 * E * sizeof(float), st>>>(
-                        (const T*)h, ldh, (const T*)wr, (const float*)corr, (int*)idx, (float*)wts, E, K, top, vec)));
+                        (const T*)h, ldh, (const T*)wr, (const float*)corr, (int*)idx, (float*)wts, E, K, top, vec,
+                        norm)));
   HIP_CHECK_LAUNCH();
 }
 
@@ -217,7 +228,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ 
                                                           const T* __restrict__ wg, const T* __restrict__ wu,
                                                           const int* __restrict__ meta, const int* __restrict__ order,
                                                           T* __restrict__ act, int E, int maxt, int top, int F, int K,
-                                                          float limit, float alpha) {
+                                                          float limit, float alpha, const float* __restrict__ pw,
+                                                          int silu) {
   __shared__ float As[TV_BK][TV_LD];
   __shared__ float Gs[TV_BK][TV_LD];
   __shared__ float Us[TV_BK][TV_LD];
@@ -253,10 +265,11 @@ __global__ __launch_bounds__(256) void moe_gate_up_kernel(const T* __restrict__ 
   for (int i = 0; i < 4; ++i) {
     const int m = ty * 4 + i;
     if (m >= rows) continue;
+    const float sw = pw ? pw[order[row0 + m]] : 1.0f;  // the pair's weight on the expert's input
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int f = n0 + tx * 4 + j;
-      if (f < F) El<T>::st(act + (int64_t)(row0 + m) * F + f, glu_clamped(ag[i][j], au[i][j], limit, alpha));
+      if (f < F) El<T>::st(act + (int64_t)(row0 + m) * F + f, glu_value(ag[i][j] * sw, au[i][j] * sw, limit, alpha, silu));
     }
   }
 }
@@ -306,13 +319,13 @@ __global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ act
 
 void launch_moe_gate_up(const void* h, int64_t ldh, const void* wg, const void* wu, const void* meta,
                         const void* order, void* act, int E, int maxt, int top, int F, int K, float limit,
-                        float alpha, int dt, hipStream_t st) {
+                        float alpha, int dt, const void* pw, int silu, hipStream_t st) {
   if (maxt <= 0) return;
   if (maxt > 65535) throw std::runtime_error("moe_gate_up: too many row tiles");
   dim3 g((F + TV_BN - 1) / TV_BN, maxt);
   DISPATCH_T(dt, T, (moe_gate_up_kernel<T><<<g, 256, 0, st>>>((const T*)h, ldh, (const T*)wg, (const T*)wu,
                                                                (const int*)meta, (const int*)order, (T*)act, E, maxt,
-                                                               top, F, K, limit, alpha)));
+                                                               top, F, K, limit, alpha, (const float*)pw, silu)));
   HIP_CHECK_LAUNCH();
 }
 
@@ -335,7 +348,7 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restric
   for (int c = threadIdx.x; c < N; c += blockDim.x) {
     float a = 0.f;
     for (int j = 0; j < top; ++j)
-      a = fmaf(wts[(int64_t)t * top + j], y[(int64_t)place[(int64_t)t * top + j] * N + c], a);
+      a = fmaf(wts ? wts[(int64_t)t * top + j] : 1.0f, y[(int64_t)place[(int64_t)t * top + j] * N + c], a);
     if (shared_) a += El<T>::ld(shared_ + (int64_t)t * lds_ + c);
     out[(int64_t)t * N + c] = a;
   }

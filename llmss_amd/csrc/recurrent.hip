@@ -6,6 +6,8 @@
 //   delta (MODE 1):  S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q
 //                    k <- k / sqrt(|k|^2 + 1e-6), q <- q / sqrt(|q|^2 + 1e-6) / sqrt(dim)
 //                    beta = sigmoid(b), g = exp(-exp(A_log[head]) softplus(a + dt_bias[head]))
+//   ssd   (MODE 2):  d = softplus(a + dt_bias[head]); S <- exp(-exp(A_log[head]) d) S + d k v^T
+//                    o = S^T q + D[head] v             (k = B, q = C of the head's group, v = the head's input x)
 //
 // Both updates act on the columns of S independently: column c needs only v[c] and the whole k and q. So a thread
 // owns one column, split over 1, 2 or 4 neighbouring lanes (32 to 128 state values in registers each) that reduce
@@ -60,6 +62,7 @@ struct RecArgs {
   int64_t ldo;
   int H, G, dim, vdim, silu_in;
   int gates_ready;  // delta: a / b already hold g / beta (delta_gates_kernel), nothing left to compute while staging
+  const float* skip;  // ssd: D [H]
 };
 
 // TQ: storage of q / k / v; TP: storage of a / b. R: state values per lane, P lanes per column. Staging: every
@@ -109,6 +112,7 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
     dtb = A.dt_bias[h];
   }
   const float qmul = MODE == 1 ? 1.0f / sqrtf((float)dim) : 1.0f;
+  const float dskip = MODE == 2 ? A.skip[h] : 0.f;
   // this thread's staged numbers: slots 0 .. REC_NE - 2 hold k / q / v entries (storage TQ), the last slot the
   // head's two per-token scalars (storage TP, threads 0 and 1). A slot without an entry points at a valid address
   // all the same, so every load is unconditional and the whole batch is in flight together.
@@ -130,7 +134,7 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
       if (c < vdim) has[k] = true, ld[k] = A.ldv, src[k] = (const TQ*)A.v + (int64_t)t0 * A.ldv + (int64_t)h * vdim + c;
     }
   }
-  const bool has_s = MODE == 1 && threadIdx.x < 2;  // thread 0: beta's input, thread 1: the decay's
+  const bool has_s = MODE >= 1 && threadIdx.x < 2;  // thread 0: beta's input (ssd: the step size's), thread 1: the decay's
   const TP* src_s = has_s ? (const TP*)A.ab + (int64_t)t0 * A.ldab + (threadIdx.x == 0 ? A.off_b : A.off_a) + h : nullptr;
   float pre[REC_CT * REC_NE];
   auto fetch = [&](int j0) {
@@ -139,7 +143,7 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
       const int64_t tj = min(j0 + jj, qlen - 1);
 #pragma unroll
       for (int k = 0; k < REC_NE - 1; ++k) pre[jj * REC_NE + k] = El<TQ>::ld(src[k] + tj * ld[k]);
-      if (MODE == 1) pre[jj * REC_NE + REC_NE - 1] = has_s ? El<TP>::ld(src_s + tj * A.ldab) : 0.f;
+      if (MODE >= 1) pre[jj * REC_NE + REC_NE - 1] = has_s ? El<TP>::ld(src_s + tj * A.ldab) : 0.f;
     }
   };
   auto put = [&]() {
@@ -157,7 +161,12 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
         float v = pre[jj * REC_NE + REC_NE - 1];
         if (A.gates_ready) {
         } else if (threadIdx.x == 0) {
-          v = 1.0f / (1.0f + expf(-v));
+          if (MODE == 2) {
+            const float z = v + dtb;
+            v = z > 20.f ? z : log1pf(expf(z));
+          } else {
+            v = 1.0f / (1.0f + expf(-v));
+          }
         } else {
           const float z = v + dtb;
           v = expf(-a_const * (z > 20.f ? z : log1pf(expf(z))));
@@ -190,6 +199,21 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
           for (int i = 0; i < 32; ++i) {
             if (d0 + c0 + i < dim) {
               S[c0 + i] = fmaf(a_const, S[c0 + i], kr[i] * vv);
+              o4[i & 3] = fmaf(S[c0 + i], qr[i], o4[i & 3]);
+            }
+          }
+        }
+      } else if (MODE == 2) {
+        const float dv = ks[2 * dimp + cols] * vv, gg = ks[2 * dimp + cols + 1];
+#pragma unroll
+        for (int c0 = 0; c0 < R; c0 += 32) {
+          float kr[32], qr[32];
+          ld32(ks + d0 + c0, kr);
+          ld32(qs + d0 + c0, qr);
+#pragma unroll
+          for (int i = 0; i < 32; ++i) {
+            if (d0 + c0 + i < dim) {
+              S[c0 + i] = fmaf(gg, S[c0 + i], kr[i] * dv);
               o4[i & 3] = fmaf(S[c0 + i], qr[i], o4[i & 3]);
             }
           }
@@ -237,6 +261,7 @@ __global__ __launch_bounds__(256) void recurrence_kernel(RecArgs A, int P, int c
       }
       float o = (o4[0] + o4[1]) + (o4[2] + o4[3]);
       o = part_sum(o, P);
+      if (MODE == 2) o = fmaf(dskip, vv, o);
       if (live && part == 0) A.out[(int64_t)(t0 + j0 + jj) * A.ldo + (int64_t)h * vdim + col] = o;
     }
   }
@@ -272,12 +297,15 @@ static void recurrence_t(const RecArgs& A, int B, hipStream_t st) {
 void launch_recurrence(int mode, const void* q, const void* k, const void* v, int64_t ldq, int64_t ldk, int64_t ldv,
                        const void* ab, int64_t ldab, int off_a, int off_b, const void* decay, const void* dt_bias,
                        void* state, const void* cu, const void* ctx, const void* sslots, void* out, int64_t ldo, int B,
-                       int H, int G, int dim, int vdim, int silu_in, int gates_ready, int dq, int dp, hipStream_t st) {
+                       int H, int G, int dim, int vdim, int silu_in, int gates_ready, int dq, int dp, const void* skip,
+                       hipStream_t st) {
   if (B == 0) return;
   if (G < 1 || H % G) throw std::runtime_error("recurrence: heads must be a multiple of the key heads");
   RecArgs A{q, k, v, ldq, ldk, ldv, ab, ldab, off_a, off_b, (const float*)decay, (const float*)dt_bias, (float*)state,
-            (const int*)cu, (const int*)ctx, (const int*)sslots, (float*)out, ldo, H, G, dim, vdim, silu_in, gates_ready};
+            (const int*)cu, (const int*)ctx, (const int*)sslots, (float*)out, ldo, H, G, dim, vdim, silu_in, gates_ready,
+            (const float*)skip};
   if (mode == 0) DISPATCH_T(dq, TQ, (recurrence_t<TQ, float, 0>(A, B, st)));
+  else if (mode == 2) DISPATCH_T(dq, TQ, DISPATCH_T(dp, TP, (recurrence_t<TQ, TP, 2>(A, B, st))));
   else DISPATCH_T(dq, TQ, DISPATCH_T(dp, TP, (recurrence_t<TQ, TP, 1>(A, B, st))));
   HIP_CHECK_LAUNCH();
 }

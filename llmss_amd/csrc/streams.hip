@@ -134,7 +134,8 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const TI* __restrict__
                                                           const TW* __restrict__ w, const float* __restrict__ state,
                                                           const int* __restrict__ cu, const int* __restrict__ ctx,
                                                           const int* __restrict__ sslots, TO* __restrict__ out,
-                                                          int64_t ldo, int B, int C, int taps, int res, int silu) {
+                                                          int64_t ldo, int B, int C, int taps, int res, int silu,
+                                                          const TW* __restrict__ bias) {
   const int t = blockIdx.x;
   const RowSeq r = row_seq(cu, ctx, B, t);  // once per workgroup: a thread walks CONV_CPT channels
   const int c_end = min(C, (int)(blockIdx.y + 1) * (int)blockDim.x * CONV_CPT);
@@ -155,6 +156,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const TI* __restrict__
       else v = state[((int64_t)slot * R + (r.j - d + R)) * C + c];
       acc = fmaf(El<TW>::ld(w + (int64_t)c * taps + k), v, acc);
     }
+    if (bias) acc += El<TW>::ld(bias + c);
     if (silu) acc = acc / (1.0f + expf(-acc));
     El<TO>::st(out + (int64_t)t * ldo + c, acc);
   }
@@ -202,7 +204,7 @@ __global__ __launch_bounds__(256) void causal_conv_strip_kernel(const TI* __rest
                                                                 const int* __restrict__ cu, const int* __restrict__ ctx,
                                                                 const int* __restrict__ sslots, TO* __restrict__ out,
                                                                 int64_t ldo, int B, int C, int taps, int res, int silu,
-                                                                int T_) {
+                                                                int T_, const TW* __restrict__ bias) {
   const int t0 = blockIdx.x * CONV_STRIP;
   const int c = (blockIdx.y * blockDim.x + threadIdx.x) * CH;
   if (c >= C) return;  // (C is a multiple of CH)
@@ -254,6 +256,10 @@ __global__ __launch_bounds__(256) void causal_conv_strip_kernel(const TI* __rest
 #pragma unroll
         for (int e = 0; e < CH; ++e) acc[e] = fmaf(wd[d][e], v[e], acc[e]);
       }
+      if (bias) {
+#pragma unroll
+        for (int e = 0; e < CH; ++e) acc[e] += El<TW>::ld(bias + c + e);
+      }
       if (silu) {
 #pragma unroll
         for (int e = 0; e < CH; ++e) acc[e] = acc[e] / (1.0f + expf(-acc[e]));
@@ -293,14 +299,14 @@ __global__ __launch_bounds__(256) void conv_tail_kernel(const TI* __restrict__ i
 template <typename TI, typename TW, typename TO>
 static void causal_conv_t(const void* in, int64_t ldi, const void* w, void* state, const void* cu, const void* ctx,
                           const void* sslots, void* out, int64_t ldo, int T_, int B, int C, int taps, int res,
-                          int silu, hipStream_t st) {
+                          int silu, const void* bias, hipStream_t st) {
   if (T_ >= 256 && T_ >= 8 * B && taps <= 9) {  // portions of eight rows and more on average
     const auto al16 = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
     const bool four = C % 4 == 0 && ldi % 4 == 0 && ldo % 4 == 0 && al16(in) && al16(out) && al16(state);
 #define LAUNCH_STRIP(RMAX_, CH_)                                                                                    \
   causal_conv_strip_kernel<TI, TW, TO, RMAX_, CH_><<<g, 256, 0, st>>>(                                              \
       (const TI*)in, ldi, (const TW*)w, (const float*)state, (const int*)cu, (const int*)ctx, (const int*)sslots,   \
-      (TO*)out, ldo, B, C, taps, res, silu, T_)
+      (TO*)out, ldo, B, C, taps, res, silu, T_, (const TW*)bias)
     if (four) {
       dim3 g((T_ + CONV_STRIP - 1) / CONV_STRIP, (C / 4 + 255) / 256);
       if (taps <= 4) LAUNCH_STRIP(3, 4);
@@ -315,7 +321,7 @@ static void causal_conv_t(const void* in, int64_t ldi, const void* w, void* stat
     dim3 g(T_, (C + 256 * CONV_CPT - 1) / (256 * CONV_CPT));
     causal_conv_kernel<TI, TW, TO><<<g, 256, 0, st>>>((const TI*)in, ldi, (const TW*)w, (const float*)state,
                                                       (const int*)cu, (const int*)ctx, (const int*)sslots, (TO*)out,
-                                                      ldo, B, C, taps, res, silu);
+                                                      ldo, B, C, taps, res, silu, (const TW*)bias);
   }
   if (taps > 1) {
     dim3 g2(B, (C + 255) / 256);
@@ -327,47 +333,56 @@ static void causal_conv_t(const void* in, int64_t ldi, const void* w, void* stat
 // di / dw / dout: storage types of the input, the weights and the output (0 bf16, 1 fp32)
 void launch_causal_conv(const void* in, int64_t ldi, const void* w, void* state, const void* cu, const void* ctx,
                         const void* sslots, void* out, int64_t ldo, int T_, int B, int C, int taps, int res, int silu,
-                        int di, int dw, int dout, hipStream_t st) {
+                        int di, int dw, int dout, const void* bias, hipStream_t st) {
   if (T_ == 0 || B == 0) return;
   if (taps < 1 || taps - 1 > MAX_TAIL) throw std::runtime_error("causal_conv: 1 to 17 taps");
   if ((C + 255) / 256 > 65535) throw std::runtime_error("causal_conv: too many channels");
   DISPATCH_T(di, TI, DISPATCH_T(dw, TW, DISPATCH_T(dout, TO, (causal_conv_t<TI, TW, TO>(
-      in, ldi, w, state, cu, ctx, sslots, out, ldo, T_, B, C, taps, res, silu, st)))));
+      in, ldi, w, state, cu, ctx, sslots, out, ldo, T_, B, C, taps, res, silu, bias, st)))));
   HIP_CHECK_LAUNCH();
 }
 
 // out[t, g * n + i] = c * o[t, g * n + i] / sqrt(mean_i(o[t, g, :]^2) + eps) * w[i] * act(gate[t, g * n + i])
-// act 0: sigmoid, 1: silu. o fp32; gate, w and out in the storage type.
+// act 0: sigmoid, 1: silu. o fp32; gate, w and out in the storage type. wfull: w holds a weight per column, w[g * n +
+// i]. first: the gate comes before the norm, out = c * u / sqrt(mean(u^2) + eps) * w with u = o * act(gate).
 template <typename T>
 __global__ __launch_bounds__(256) void gated_group_norm_kernel(const float* __restrict__ o, int64_t ldo,
                                                                const T* __restrict__ gate, int64_t ldg,
                                                                const T* __restrict__ w, float eps, int act, float c,
-                                                               T* __restrict__ out, int64_t ldout, int n) {
+                                                               T* __restrict__ out, int64_t ldout, int n, int wfull,
+                                                               int first) {
   __shared__ float red[32];
   const int t = blockIdx.x, g = blockIdx.y;
   const float* row = o + (int64_t)t * ldo + (int64_t)g * n;
-  float ss = 0.f;
-  for (int i = threadIdx.x; i < n; i += blockDim.x) ss = fmaf(row[i], row[i], ss);
-  ss = block_sum(ss, red);
-  const float inv = c / sqrtf(ss / (float)n + eps);
   const T* gr = gate + (int64_t)t * ldg + (int64_t)g * n;
-  T* dst = out + (int64_t)t * ldout + (int64_t)g * n;
-  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+  const T* wr = wfull ? w + (int64_t)g * n : w;
+  auto gate_of = [&](int i) {
     const float z = El<T>::ld(gr + i);
     const float sg = 1.0f / (1.0f + expf(-z));
-    El<T>::st(dst + i, row[i] * inv * El<T>::ld(w + i) * (act ? z * sg : sg));
+    return act ? z * sg : sg;
+  };
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const float u = first ? row[i] * gate_of(i) : row[i];
+    ss = fmaf(u, u, ss);
   }
+  ss = block_sum(ss, red);
+  const float inv = c / sqrtf(ss / (float)n + eps);
+  T* dst = out + (int64_t)t * ldout + (int64_t)g * n;
+  for (int i = threadIdx.x; i < n; i += blockDim.x)
+    El<T>::st(dst + i, row[i] * inv * El<T>::ld(wr + i) * gate_of(i));
 }
 
 void launch_gated_group_norm(const void* o, int64_t ldo, const void* gate, int64_t ldg, const void* w, float eps,
-                             int act, float c, void* out, int64_t ldout, int T_, int groups, int n, int dt,
-                             hipStream_t st) {
+                             int act, float c, void* out, int64_t ldout, int T_, int groups, int n, int dt, int wfull,
+                             int first, hipStream_t st) {
   if (T_ == 0) return;
   if (groups > 65535) throw std::runtime_error("gated_group_norm: too many groups");
   dim3 g(T_, groups);
   const int threads = n >= 256 ? 256 : ((n + 63) / 64) * 64;
   DISPATCH_T(dt, T, (gated_group_norm_kernel<T><<<g, threads, 0, st>>>((const float*)o, ldo, (const T*)gate, ldg,
-                                                                        (const T*)w, eps, act, c, (T*)out, ldout, n)));
+                                                                        (const T*)w, eps, act, c, (T*)out, ldout, n,
+                                                                        wfull, first)));
   HIP_CHECK_LAUNCH();
 }
 

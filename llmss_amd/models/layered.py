@@ -296,9 +296,10 @@ class PoolAttention:
         q = ops.rope_pairs_cache(proj, c["q"], c["k"], c["v"], cs, kc, vc, inp.slots, spec.heads, spec.kv_heads,
                                  spec.dim, spec.vdim)
         kp, vp = pooled.get("kp"), pooled.get("vp")
-        if spec.pool:
-            ops.pool_update(kc, vc, kp, vp, inp.block_tables, cu, inp.ctx_lens, spec.pool)
         single = inp.kind == "decode"
+        if spec.pool:
+            ops.pool_update(kc, vc, kp, vp, inp.block_tables, cu, inp.ctx_lens, spec.pool,
+                            max_qlen=1 if single else max(1, inp.max_seqlen))
         y = ops.pool_window_attn(q, kc, vc, kp, vp, inp.block_tables, cu, inp.ctx_lens, W.pb, spec.heads,
                                  spec.kv_heads, spec.dim, spec.vdim, spec.scale, spec.window, spec.pool, dt,
                                  max_qlen=1 if single else max(1, inp.max_seqlen),

@@ -822,10 +822,11 @@ class MoEPending:
     pair, ``wts`` [T, top], ``shared`` [T, N] or None. resid_add_norm takes it as its fp32 addend and combines while
     it adds to the stream."""
 
-    __slots__ = ("y", "place", "wts", "shared")
+    __slots__ = ("y", "place", "wts", "shared", "top")
 
-    def __init__(self, y, place, wts, shared):
+    def __init__(self, y, place, wts, shared, top=None):
         self.y, self.place, self.wts, self.shared = y, place, wts, shared
+        self.top = top if top is not None else wts.shape[1]  # wts None: the outputs are summed unweighted
 
 
 def resid_add_norm(x, a, b, w, woff, eps, out_dtype, want_y=True):
@@ -837,6 +838,7 @@ def resid_add_norm(x, a, b, w, woff, eps, out_dtype, want_y=True):
         _check(a.shape[0] == T, "a rows")
     pend = b if isinstance(b, MoEPending) else None
     if pend is not None:
+        _check(pend.wts is not None, "resid_add_norm combines weighted expert outputs")
         top = pend.wts.shape[1]
         _check(pend.y.shape == (T * top, H) and pend.y.is_contiguous() and pend.place.numel() == T * top
                and pend.wts.shape[0] == T, "pending expert outputs do not fit the stream")
@@ -1015,7 +1017,7 @@ def glu_clamp(gu, F, limit, alpha):
     return out
 
 
-def moe_route(z, corr, top):
+def moe_route(z, corr, top, normalize=True):
     T, E = z.shape
     _rows(z, "z", dtype=torch.float32)
     _check(z.is_contiguous(), "router logits contiguous")
@@ -1025,20 +1027,20 @@ def moe_route(z, corr, top):
                "correction fp32 [E]")
     idx = torch.empty(T, top, dtype=torch.int32, device=z.device)
     wts = torch.empty(T, top, dtype=torch.float32, device=z.device)
-    lib().moe_route(z.data_ptr(), _ptr(corr), idx.data_ptr(), wts.data_ptr(), T, E, top, _stream())
+    lib().moe_route(z.data_ptr(), _ptr(corr), idx.data_ptr(), wts.data_ptr(), T, E, top, int(bool(normalize)), _stream())
     return idx, wts
 
 
 ROUTER_FUSED_MAX_ROWS = 1024  # steps of at most this many tokens compute logits and routing in one launch
 
 
-def moe_router(h, router, corr, top):
+def moe_router(h, router, corr, top, normalize=True):
     """(idx [T, top] int32, wts [T, top] fp32) from the layer input: fp32 router logits, then moe_route. Few rows (a
     decode step): one fused launch; a prompt: the matrix-core GEMM with fp32 output, then moe_route."""
     T, K = h.shape
     E = router.shape[0]
     if T > ROUTER_FUSED_MAX_ROWS:
-        return moe_route(linear_f(h, router, torch.float32), corr, top)
+        return moe_route(linear_f(h, router, torch.float32), corr, top, normalize)
     _rows(h, "h")
     _check(router.dtype == h.dtype and router.is_contiguous() and router.shape == (E, K) and router.is_cuda,
            "router [E, K] in h's storage type")
@@ -1049,12 +1051,15 @@ def moe_router(h, router, corr, top):
     idx = torch.empty(T, top, dtype=torch.int32, device=h.device)
     wts = torch.empty(T, top, dtype=torch.float32, device=h.device)
     lib().moe_router(h.data_ptr(), h.stride(0), router.data_ptr(), _ptr(corr), idx.data_ptr(), wts.data_ptr(), T, E, K,
-                     top, _dt(h, "h"), _stream())
+                     top, _dt(h, "h"), int(bool(normalize)), _stream())
     return idx, wts
 
 
-def moe_experts(h, idx, wts, gate, up, down, limit, alpha, shared=None, combine=True):
-    """``combine=False``: leave the weighting and summing to resid_add_norm (returns a :class:`MoEPending`)."""
+def moe_experts(h, idx, wts, gate, up, down, limit, alpha, shared=None, combine=True, act="glu_clamp",
+                weight_input=False):
+    """``combine=False``: leave the weighting and summing to the next residual add (returns a :class:`MoEPending`).
+    ``weight_input``: the weights scale the two input products in the gate / up epilogue (the experts have no
+    biases), and the outputs are summed plainly (``MoEPending.wts`` is None)."""
     T, K = h.shape
     E, F, _ = gate.shape
     N = down.shape[1]
@@ -1080,22 +1085,25 @@ def moe_experts(h, idx, wts, gate, up, down, limit, alpha, shared=None, combine=
     meta = torch.empty(1 + (E + 1) + 2 * maxt, dtype=torch.int32, device=dev)
     order = torch.empty(P, dtype=torch.int32, device=dev)
     place = torch.empty(P, dtype=torch.int32, device=dev)
-    act = torch.empty(P, F, dtype=h.dtype, device=dev)
+    act_ = torch.empty(P, F, dtype=h.dtype, device=dev)
     y = torch.empty(P, N, dtype=torch.float32, device=dev)
+    _check(act in ("glu_clamp", "silu"), "expert activation: glu_clamp or silu")
+    pw, silu = (wts.data_ptr() if weight_input else 0), int(act == "silu")
     L = lib()
     st = _stream()
     L.moe_group(idx.data_ptr(), P, E, maxt, meta.data_ptr(), order.data_ptr(), place.data_ptr(), rows, st)
     if h.dtype == torch.bfloat16:  # matrix cores (csrc/gemm_tile.hip)
         L.moe_gate_up_tile(h.data_ptr(), h.stride(0), gate.data_ptr(), up.data_ptr(), meta.data_ptr(),
-                           order.data_ptr(), act.data_ptr(), E, maxt, top, F, K, float(limit), float(alpha), rows, st)
-        L.moe_down_tile(act.data_ptr(), down.data_ptr(), meta.data_ptr(), y.data_ptr(), E, maxt, N, F, rows, st)
+                           order.data_ptr(), act_.data_ptr(), E, maxt, top, F, K, float(limit), float(alpha), rows, pw,
+                           silu, st)
+        L.moe_down_tile(act_.data_ptr(), down.data_ptr(), meta.data_ptr(), y.data_ptr(), E, maxt, N, F, rows, st)
     else:
         L.moe_gate_up(h.data_ptr(), h.stride(0), gate.data_ptr(), up.data_ptr(), meta.data_ptr(), order.data_ptr(),
-                      act.data_ptr(), E, maxt, top, F, K, float(limit), float(alpha), dt, st)
-        L.moe_down(act.data_ptr(), down.data_ptr(), meta.data_ptr(), y.data_ptr(), E, maxt, N, F, dt, st)
+                      act_.data_ptr(), E, maxt, top, F, K, float(limit), float(alpha), dt, pw, silu, st)
+        L.moe_down(act_.data_ptr(), down.data_ptr(), meta.data_ptr(), y.data_ptr(), E, maxt, N, F, dt, st)
     if not combine:
-        return MoEPending(y, place, wts, shared)
-    L.moe_combine(y.data_ptr(), place.data_ptr(), wts.data_ptr(), _ptr(shared),
+        return MoEPending(y, place, None if weight_input else wts, shared, top)
+    L.moe_combine(y.data_ptr(), place.data_ptr(), 0 if weight_input else wts.data_ptr(), _ptr(shared),
                   shared.stride(0) if shared is not None else 0, out.data_ptr(), T, N, top, dt, st)
     return out
 
@@ -1157,7 +1165,7 @@ def stream_add_norm(x, y, mix, outw, c, inw, w, eps, rms, out_dtype):
     return h
 
 
-def causal_conv(x, w, state, cu, ctx_lens, state_slots, residual, silu, out_dtype):
+def causal_conv(x, w, state, cu, ctx_lens, state_slots, residual, silu, out_dtype, bias=None):
     T, C = x.shape
     _rows(x, "x")
     taps = w.shape[1]
@@ -1169,18 +1177,25 @@ def causal_conv(x, w, state, cu, ctx_lens, state_slots, residual, silu, out_dtyp
     if taps > 1:
         _f32c(state, "state")
         _check(state.dim() == 3 and tuple(state.shape[1:]) == (taps - 1, C), "state [slots, taps - 1, C]")
+    if bias is not None:
+        _check(bias.dtype == w.dtype and bias.is_contiguous() and bias.numel() == C and bias.is_cuda, "conv bias [C]")
     out = torch.empty(T, C, dtype=out_dtype, device=x.device)
     lib().causal_conv(x.data_ptr(), x.stride(0), w.data_ptr(), _ptr(state) if taps > 1 else 0, cu.data_ptr(),
                       ctx_lens.data_ptr(), state_slots.data_ptr(), out.data_ptr(), C, T, B, C, taps,
-                      int(bool(residual)), int(bool(silu)), _dt(x, "x"), _dt(w, "w"), _DT[out_dtype], _stream())
+                      int(bool(residual)), int(bool(silu)), _dt(x, "x"), _dt(w, "w"), _DT[out_dtype], _ptr(bias),
+                      _stream())
     return out
 
 
-def gated_group_norm(o, gate, w, eps, act, c, out=None, out_dtype=None):
+def gated_group_norm(o, gate, w, eps, act, c, out=None, out_dtype=None, groups=0, gate_first=False):
     T, N = o.shape
     _rows(o, "o", dtype=torch.float32)
-    n = w.numel()
-    _check(N % n == 0 and w.is_contiguous(), "the group size (len(w)) must divide the row")
+    if groups:
+        _check(N % groups == 0 and w.numel() == N and w.is_contiguous(), "a weight per column, groups dividing the row")
+        n = N // groups
+    else:
+        n = w.numel()
+        _check(N % n == 0 and w.is_contiguous(), "the group size (len(w)) must divide the row")
     _rows(gate, "gate", N)
     if out is None:
         out = torch.empty(T, N, dtype=out_dtype, device=o.device)
@@ -1188,7 +1203,7 @@ def gated_group_norm(o, gate, w, eps, act, c, out=None, out_dtype=None):
     _check(gate.dtype == w.dtype == out.dtype and gate.shape[0] == T and out.shape[0] == T, "gate / w / out types, rows")
     lib().gated_group_norm(o.data_ptr(), o.stride(0), gate.data_ptr(), gate.stride(0), w.data_ptr(), float(eps),
                            {"sigmoid": 0, "silu": 1}[act], float(c), out.data_ptr(), out.stride(0), T, N // n, n,
-                           _dt(w, "w"), _stream())
+                           _dt(w, "w"), int(bool(groups)), int(bool(gate_first)), _stream())
     return out
 
 
@@ -1233,7 +1248,7 @@ def decay_recurrence(q, k, v, decay, state, cu, ctx_lens, state_slots, heads, di
         lib().recurrence(0, q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), v.stride(0), 0, 0, 0, 0,
                          decay.data_ptr(), 0, state.data_ptr(), cu.data_ptr(), ctx_lens.data_ptr(),
                          state_slots.data_ptr(), out.data_ptr(), heads * vdim, B, heads, heads, dim, vdim,
-                         int(bool(silu_in)), 0, _dt(q, "q"), 0, _stream())
+                         int(bool(silu_in)), 0, _dt(q, "q"), 0, 0, _stream())
     return out
 
 
@@ -1258,7 +1273,7 @@ def delta_recurrence(q, k, v, a, b_, A_log, dt_bias, state, cu, ctx_lens, state_
         lib().recurrence(1, q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), k.stride(0), v.stride(0),
                          a.data_ptr(), a.stride(0), 0, int(off_b), A_log.data_ptr(), dt_bias.data_ptr(),
                          state.data_ptr(), cu.data_ptr(), ctx_lens.data_ptr(), state_slots.data_ptr(), out.data_ptr(),
-                         heads * vdim, B, heads, kv_heads, dim, vdim, 0, ready, _dt(q, "q"), _dt(a, "a"), _stream())
+                         heads * vdim, B, heads, kv_heads, dim, vdim, 0, ready, _dt(q, "q"), _dt(a, "a"), 0, _stream())
     return out
 
 
@@ -1447,3 +1462,166 @@ def diff_combine(O, lam, eps, mult, heads, kv_heads, vdim, out_dtype):
     lib().diff_combine(O.data_ptr(), float(lam), float(eps), float(mult), y.data_ptr(), y.stride(0), T, heads,
                        kv_heads, vdim, _DT[out_dtype], _stream())
     return y
+
+
+# ------------------- blocks normed on both sides / token input / windowed sigmoid attention with pooled blocks / SSD
+def sandwich_add_norm(x, y, r, rb, wpost, eps, add, wnext, out_dtype):
+    """``y``: rows in the storage type, or a :class:`MoEPending` (combined while it is read)."""
+    T, W = x.shape
+    _rows(x, "x", dtype=torch.float32)
+    _check(x.is_contiguous(), "x contiguous")
+    _check(out_dtype in _DT, "storage type bf16 / fp32")
+    pend = y if isinstance(y, MoEPending) else None
+    sh = None
+    if pend is not None:
+        _check(pend.y.shape == (T * pend.top, W) and pend.y.is_contiguous() and pend.place.numel() == T * pend.top,
+               "pending expert outputs do not fit the stream")
+        if pend.wts is not None:
+            _check(tuple(pend.wts.shape) == (T, pend.top) and pend.wts.is_contiguous(), "pending weights [T, top]")
+        sh = pend.shared
+        if sh is not None:
+            _rows(sh, "shared", W, out_dtype)
+    elif y is not None:
+        _rows(y, "y", W, out_dtype)
+        _check(y.shape[0] == T, "y rows")
+    if y is not None:
+        _f32c(wpost, "wpost")
+        _check(wpost.numel() == W, "wpost [W]")
+        if r is not None:
+            _rows(r, "r", W, out_dtype)
+            _f32c(rb, "rb")
+            _check(r.shape[0] == T and rb.numel() == W, "gate logits [T, W], bias [W]")
+    if add is not None:
+        _f32c(add, "add")
+        _check(tuple(add.shape) == (T, W), "add fp32 [T, W]")
+    h = None
+    if wnext is not None:
+        _f32c(wnext, "wnext")
+        _check(wnext.numel() == W, "wnext [W]")
+        h = torch.empty(T, W, dtype=out_dtype, device=x.device)
+    dense = y if pend is None else None
+    lib().sandwich_add_norm(x.data_ptr(), _ptr(dense), dense.stride(0) if dense is not None else 0,
+                            _ptr(pend.y) if pend else 0, _ptr(pend.place) if pend else 0,
+                            _ptr(pend.wts) if pend else 0, pend.top if pend else 0, _ptr(sh),
+                            sh.stride(0) if sh is not None else 0, _ptr(r) if y is not None else 0,
+                            r.stride(0) if (r is not None and y is not None) else 0, _ptr(rb), _ptr(wpost), _ptr(add),
+                            _ptr(wnext), _ptr(h), W, float(eps), T, W, _DT[out_dtype], _stream())
+    return h
+
+
+def token_side_add(x, ids, table, col0, gate_w, proj_w, norm_w, eps, add, wnext, out_dtype):
+    T, W = x.shape
+    _rows(x, "x", dtype=torch.float32)
+    _check(x.is_contiguous(), "x contiguous")
+    d = gate_w.shape[0]
+    _check(ids.dtype == torch.int64 and ids.is_contiguous() and ids.is_cuda and ids.numel() == T, "ids: int64 [T] cuda")
+    _rows(table, "token table", dtype=out_dtype)
+    _check(0 <= col0 and col0 + d <= table.shape[1], "the layer's columns lie outside the token table")
+    _check(gate_w.dtype == out_dtype and gate_w.is_contiguous() and tuple(gate_w.shape) == (d, W) and gate_w.is_cuda,
+           "gate [d, W] in the storage type")
+    _check(proj_w.dtype == out_dtype and proj_w.is_contiguous() and tuple(proj_w.shape) == (W, d) and proj_w.is_cuda,
+           "proj [W, d] in the storage type")
+    _f32c(norm_w, "norm_w")
+    _check(norm_w.numel() == W, "norm_w [W]")
+    if add is not None:
+        _f32c(add, "add")
+        _check(tuple(add.shape) == (T, W), "add fp32 [T, W]")
+    h = None
+    if wnext is not None:
+        _f32c(wnext, "wnext")
+        _check(wnext.numel() == W, "wnext [W]")
+        h = torch.empty(T, W, dtype=out_dtype, device=x.device)
+    lib().token_side_add(x.data_ptr(), ids.data_ptr(), table.data_ptr(), table.stride(0), table.shape[0], int(col0), d,
+                         gate_w.data_ptr(), proj_w.data_ptr(), norm_w.data_ptr(), _ptr(add), _ptr(wnext), _ptr(h), W,
+                         float(eps), T, W, _DT[out_dtype], _stream())
+    return h
+
+
+def rope_pairs_cache(proj, off_q, off_k, off_v, cs, k_cache, v_cache, slots, heads, kv_heads, dim, vdim):
+    T = proj.shape[0]
+    _rows(proj, "proj")
+    nq, nk, nv = heads * dim, kv_heads * dim, kv_heads * vdim
+    _check(min(off_q, off_k, off_v) >= 0 and max(off_q + nq, off_k + nk, off_v + nv) <= proj.shape[1],
+           "q / k / v columns outside the projection")
+    for c, n, nm in ((k_cache, nk, "k cache"), (v_cache, nv, "v cache")):
+        _check(c.dtype == proj.dtype and c.is_contiguous() and c.dim() == 3 and c.shape[2] == n,
+               f"{nm} [blocks, block_size, {n}] in the model's storage type")
+    _check(slots.dtype == torch.int64 and slots.is_contiguous() and slots.is_cuda and slots.numel() == T, "slots")
+    rdims = 0
+    if cs is not None:
+        _f32c(cs, "angles")
+        _check(cs.dim() == 3 and cs.shape[0] == T and cs.shape[2] == 2 and 2 * cs.shape[1] <= dim,
+               "angles [T, rotated dims / 2, 2], rotated dims <= dim")
+        rdims = 2 * cs.shape[1]
+    q = torch.empty(T, nq, dtype=torch.float32, device=proj.device)
+    lib().rope_pairs_cache(proj.data_ptr(), proj.stride(0), int(off_q), int(off_k), int(off_v), _ptr(cs), rdims,
+                           q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), slots.data_ptr(), T, heads, kv_heads,
+                           dim, vdim, _dt(proj, "proj"), _stream())
+    return q
+
+
+def _pool_caches(k_cache, v_cache, kp_cache, vp_cache, pool):
+    _check(k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dtype == v_cache.dtype and k_cache.dim() == 3
+           and v_cache.dim() == 3 and k_cache.shape[:2] == v_cache.shape[:2] and k_cache.is_cuda,
+           "k / v cache [blocks, block_size, n]")
+    if not pool:
+        return 0
+    bs = k_cache.shape[1]
+    per = -(-bs // pool)
+    for c, full, nm in ((kp_cache, k_cache, "pooled keys"), (vp_cache, v_cache, "pooled values")):
+        _f32c(c, nm)
+        _check(tuple(c.shape) == (full.shape[0], per, full.shape[2]), f"{nm} fp32 [blocks, ceil(block_size / pool), n]")
+    return per
+
+
+def pool_update(k_cache, v_cache, kp_cache, vp_cache, block_tables, cu, ctx_lens, pool, max_qlen=0):
+    """``max_qlen``: the step's longest portion (known on the host; bounds the blocks a portion can complete)."""
+    per = _pool_caches(k_cache, v_cache, kp_cache, vp_cache, pool)
+    B = cu.numel() - 1
+    _i32(cu, "cu")
+    _i32(ctx_lens, "ctx_lens", B)
+    _i32(block_tables, "block_tables")
+    _check(block_tables.dim() == 2 and block_tables.shape[0] >= B and pool >= 1 and max_qlen >= 1, "block tables, pool")
+    lib().pool_update(k_cache.data_ptr(), v_cache.data_ptr(), kp_cache.data_ptr(), vp_cache.data_ptr(),
+                      block_tables.data_ptr(), block_tables.shape[1], cu.data_ptr(), ctx_lens.data_ptr(), B,
+                      int(max_qlen), k_cache.shape[2], v_cache.shape[2], k_cache.shape[1], int(pool), per,
+                      _dt(k_cache, "k cache"), _stream())
+
+
+def pool_window_attn(q, k_cache, v_cache, kp_cache, vp_cache, block_tables, cu, ctx_lens, pb, heads, kv_heads, dim,
+                     vdim, scale, window, pool, out_dtype, max_qlen=0, num_decode=0):
+    T = q.shape[0]
+    _rows(q, "q", heads * dim, torch.float32)
+    _check(q.is_contiguous(), "q contiguous")
+    per = _pool_caches(k_cache, v_cache, kp_cache, vp_cache, pool)
+    _check(k_cache.shape[2] == kv_heads * dim and v_cache.shape[2] == kv_heads * vdim, "cache rows: kv_heads * dim | vdim")
+    B = cu.numel() - 1
+    _i32(cu, "cu")
+    _i32(ctx_lens, "ctx_lens", B)
+    _i32(block_tables, "block_tables")
+    _check(block_tables.dim() == 2 and block_tables.shape[0] >= B, "block tables [B, blocks]")
+    _f32c(pb, "pb")
+    _check(pb.numel() == heads and out_dtype in _DT, "pb [heads]; out bf16 / fp32")
+    out = torch.empty(T, heads * vdim, dtype=out_dtype, device=q.device)
+    lib().pool_window_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _ptr(kp_cache) if pool else 0,
+                           _ptr(vp_cache) if pool else 0, block_tables.data_ptr(), block_tables.shape[1], cu.data_ptr(),
+                           ctx_lens.data_ptr(), pb.data_ptr(), out.data_ptr(), int(out_dtype == torch.float32), T, B,
+                           heads, kv_heads, dim, vdim, k_cache.shape[1], float(scale), int(window), int(pool), per,
+                           _dt(k_cache, "k cache"), _stream())
+    return out
+
+
+def ssd_recurrence(x, Bm, Cm, dt, A_log, dt_bias, D, state, cu, ctx_lens, state_slots, heads, groups, N, vdim):
+    """The state-space scan on the matrix-state recurrence kernel: keys = B, queries = C (one per group), values = x."""
+    T, B, out = _rec_common(Cm, Bm, x, state, cu, ctx_lens, state_slots, heads, groups, N, vdim)
+    for t, nm in ((A_log, "A_log"), (dt_bias, "dt_bias"), (D, "D")):
+        _f32c(t, nm)
+        _check(t.numel() == heads, f"{nm} [heads]")
+    _rows(dt, "dt", heads)
+    _check(dt.shape[0] == T, "dt rows")
+    if T:
+        lib().recurrence(2, Cm.data_ptr(), Bm.data_ptr(), x.data_ptr(), Cm.stride(0), Bm.stride(0), x.stride(0),
+                         dt.data_ptr(), dt.stride(0), 0, 0, A_log.data_ptr(), dt_bias.data_ptr(), state.data_ptr(),
+                         cu.data_ptr(), ctx_lens.data_ptr(), state_slots.data_ptr(), out.data_ptr(), heads * vdim, B,
+                         heads, groups, N, vdim, 0, 0, _dt(x, "x"), _dt(dt, "dt"), D.data_ptr(), _stream())
+    return out

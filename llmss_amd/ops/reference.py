@@ -1021,10 +1021,10 @@ def pool_slot(block_tables, b: int, blk: int, pool: int, bs: int, per: int):
     return int(block_tables[b, p // bs]) * per + (p % bs) // pool
 
 
-def pool_update(k_cache, v_cache, kp_cache, vp_cache, block_tables, cu, ctx_lens, pool: int):
+def pool_update(k_cache, v_cache, kp_cache, vp_cache, block_tables, cu, ctx_lens, pool: int, max_qlen: int = 0):
     """Mean key and mean value (fp32) of every block of ``pool`` positions whose last position the step has just
     written, from the cached rows of the block: kp_cache / vp_cache fp32 [blocks, ceil(block_size / pool), kv_heads *
-    dim | vdim], row :func:`pool_slot`."""
+    dim | vdim], row :func:`pool_slot`. ``max_qlen`` (the step's longest portion) only sizes the GPU kernel's grid."""
     bs, per = k_cache.shape[1], kp_cache.shape[1]
     nk, nv = k_cache.shape[2], v_cache.shape[2]
     for b, _, n, p0 in _seq_rows(cu, ctx_lens):

@@ -49,11 +49,11 @@ def window_pool_attention(q, k, v, pb, scale, size, pool):
         g = h // (H // G)
         for i in range(T):
             keys, vals = [], []
-            for j in range(max(0, i - size + 1), i + 1):
+            for j in range(max(0, i - size + 1) if size else 0, i + 1):
                 keys.append(k[j, g])
                 vals.append(v[j, g])
             b = 0
-            while b * pool + pool - 1 <= i - size:
+            while size and pool and b * pool + pool - 1 <= i - size:
                 keys.append(k[b * pool:(b + 1) * pool, g].mean(0))
                 vals.append(v[b * pool:(b + 1) * pool, g].mean(0))
                 b += 1
@@ -73,7 +73,8 @@ def attention_mixer(w, p, m, h):
     if rot and rot.get("dims"):
         q = rotate_pairs(q, pos, rot["dims"], rot["base"])
         k = rotate_pairs(k, pos, rot["dims"], rot["base"])
-    o = window_pool_attention(q, k, v, w[p + "pb"], m["scale"], m["mask"]["size"], m["mask"]["pool"])
+    mask = m.get("mask") or {}
+    o = window_pool_attention(q, k, v, w[p + "pb"], m["scale"], mask.get("size", 0), mask.get("pool", 0))
     return o.reshape(T, H * vdim) @ w[p + "o"].T
 
 
@@ -143,6 +144,17 @@ def moe(w, p, f, h):
     return out
 
 
+def gated_post_norm(y, h, rg, rgb, normb, ls, eps):
+    """What a sublayer adds to the residual: its result y times sigmoid(rg h + rgb), RMS-normed with weight normb,
+    times the layer scale ls."""
+    return rms(y * torch.sigmoid(h @ rg.T + rgb), eps) * normb * ls
+
+
+def token_side(x, e, gate, proj, norm, eps):
+    """What the token input adds: e [T, d] the layer's slice of the token table's rows."""
+    return rms((gelu_tanh(x @ gate.T) * e) @ proj.T, eps) * norm
+
+
 def layer_runs(cfg):
     """Layer indices in the order they run: layers start .. stop - 1 ``times`` times in a row. Second item: whether
     the embedding output is added right before this run."""
@@ -176,20 +188,16 @@ def forward(cfg, weights, tokens, taps=None):
             y = mamba2_mixer(w, p + "mix.", L["mixer"], h, eps)
         else:
             raise ValueError(L["type"])
-        y = y * torch.sigmoid(h @ w[p + "rg1"].T + w[p + "rg1.b"])
-        x = x + rms(y, eps) * w[p + "norm1b"] * w[p + "ls1"]
+        x = x + gated_post_norm(y, h, w[p + "rg1"], w[p + "rg1.b"], w[p + "norm1b"], w[p + "ls1"], eps)
         if L.get("mlp"):
             h = rms(x, eps) * w[p + "norm2"]
             f = L["mlp"]
             y = gated_mlp(w, p + "mlp.", h) if f["kind"] == "dense" else moe(w, p + "mlp.", f, h)
-            y = y * torch.sigmoid(h @ w[p + "rg2"].T + w[p + "rg2.b"])
-            x = x + rms(y, eps) * w[p + "norm2b"] * w[p + "ls2"]
+            x = x + gated_post_norm(y, h, w[p + "rg2"], w[p + "rg2.b"], w[p + "norm2b"], w[p + "ls2"], eps)
         if side:
             d = side["dim"]
             e = w["side.embed"][tok][:, i * d:(i + 1) * d]
-            g = gelu_tanh(x @ w[p + "side.gate"].T) * e
-            y = g @ w[p + "side.proj"].T
-            x = x + rms(y, eps) * w[p + "side.norm"]
+            x = x + token_side(x, e, w[p + "side.gate"], w[p + "side.proj"], w[p + "side.norm"], eps)
         if taps is not None:
             taps.append(x.clone())
     h = rms(x, eps) * w["final.norm"]
