@@ -48,17 +48,15 @@ def window_pool_attention(q, k, v, pb, scale, size, pool):
     for h in range(H):
         g = h // (H // G)
         for i in range(T):
-            keys, vals = [], []
-            for j in range(max(0, i - size + 1) if size else 0, i + 1):
-                keys.append(k[j, g])
-                vals.append(v[j, g])
+            keys = [k[j, g] for j in range(max(0, i - size + 1) if size else 0, i + 1)]
+            vals = [v[j, g] for j in range(max(0, i - size + 1) if size else 0, i + 1)]
             b = 0
             while size and pool and b * pool + pool - 1 <= i - size:
                 keys.append(k[b * pool:(b + 1) * pool, g].mean(0))
                 vals.append(v[b * pool:(b + 1) * pool, g].mean(0))
                 b += 1
-            for kk, vv in zip(keys, vals):
-                out[i, h] += torch.sigmoid((q[i, h] * kk).sum() * scale + pb[h]) * vv
+            wgt = torch.sigmoid(torch.stack(keys) @ q[i, h] * scale + pb[h])
+            out[i, h] = wgt @ torch.stack(vals)
     return out
 
 
@@ -202,3 +200,11 @@ def forward(cfg, weights, tokens, taps=None):
             taps.append(x.clone())
     h = rms(x, eps) * w["final.norm"]
     return (h @ w["head"].T) * cfg.get("logit_scale", 1.0)
+
+
+def greedy(cfg, weights, prompt, n):
+    """n tokens generated greedily (the whole sequence recomputed for every token)."""
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(forward(cfg, weights, toks)[-1].argmax()))
+    return toks[len(prompt):]
