@@ -86,7 +86,22 @@ def main():
                     help="instead of the headline workload: prefill / decode throughput of the Lamisun design beside "
                          "the Llama family at equal size (bench/lamisun_compare.py), sizes by name, one GPU")
     ap.add_argument("--lamisun-kinds", default="lamisun,dense", help="which of the two models --lamisun runs")
+    ap.add_argument("--fizelix", nargs="?", const="w1024,w2048,w4096", default="",
+                    help="instead of the headline workload: prefill / decode throughput of the Fizelix design beside "
+                         "the Llama family at equal size (bench/fizelix_compare.py), sizes by name, one GPU")
+    ap.add_argument("--fizelix-kinds", default="fizelix,dense", help="which of the two models --fizelix runs")
     args = ap.parse_args()
+
+    if args.fizelix:
+        sys.path.insert(0, os.path.join(ROOT, "bench"))
+        import fizelix_compare
+
+        res = fizelix_compare.run(args.fizelix.split(","), args.batch_per_gpu, args.prompt_len, args.gen_len,
+                                  args.timisun_rounds,
+                                  lambda m: print(f"[bench] {m}", file=sys.stderr, flush=True),
+                                  kinds=tuple(args.fizelix_kinds.split(",")))
+        print(json.dumps(res), flush=True)
+        return
 
     if args.lamisun:
         sys.path.insert(0, os.path.join(ROOT, "bench"))
