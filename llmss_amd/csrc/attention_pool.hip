@@ -10,7 +10,8 @@
 //
 // Pooled row of block b of a sequence: page = block_table[(b * pool) / bs], rank (b * pool % bs) / pool inside it
 // (two blocks that start in the same page are at least `pool` positions apart, so their ranks differ); the pooled
-// caches are [pages, ceil(bs / pool), G * dim | G * vdim] fp32.
+// caches are [pages, ceil(bs / pool), G * dim | G * vdim] in the pages' storage type (the means are formed in fp32
+// and rounded once, as the keys and values themselves are when they are cached).
 #include "anytype.h"
 #include "seqrows.h"
 
@@ -63,7 +64,7 @@ __device__ __forceinline__ int64_t pool_row(const int* btr, int blk, int pool, i
 // grid (B, blocks a portion can complete): workgroup (b, n) takes block p0 / pool + n of sequence b
 template <typename T>
 __global__ __launch_bounds__(256) void pool_update_kernel(const T* __restrict__ kc, const T* __restrict__ vc,
-                                                          float* __restrict__ kp, float* __restrict__ vp,
+                                                          T* __restrict__ kp, T* __restrict__ vp,
                                                           const int* __restrict__ bt, int maxb,
                                                           const int* __restrict__ cu, const int* __restrict__ ctx,
                                                           int nk, int nv, int bs, int pool, int per) {
@@ -86,7 +87,7 @@ __global__ __launch_bounds__(256) void pool_update_kernel(const T* __restrict__ 
       const int j = blk * pool + i;
       a += El<T>::ld(src + ((int64_t)btr[j / bs] * bs + j % bs) * n + cc);
     }
-    (isk ? kp : vp)[dst * n + cc] = a * inv;
+    El<T>::st((isk ? kp : vp) + dst * n + cc, a * inv);
   }
 }
 
@@ -97,7 +98,7 @@ void launch_pool_update(const void* kc, const void* vc, void* kp, void* vp, cons
   const int ny = max_qlen / pool + 1;
   if (B > 65535 * 32 || ny > 65535) throw std::runtime_error("pool_update: grid too large");
   dim3 g(B, ny);
-  DISPATCH_T(dt, T, (pool_update_kernel<T><<<g, 256, 0, st>>>((const T*)kc, (const T*)vc, (float*)kp, (float*)vp,
+  DISPATCH_T(dt, T, (pool_update_kernel<T><<<g, 256, 0, st>>>((const T*)kc, (const T*)vc, (T*)kp, (T*)vp,
                                                               (const int*)bt, maxb, (const int*)cu, (const int*)ctx,
                                                               nk, nv, bs, pool, per)));
   HIP_CHECK_LAUNCH();
@@ -110,8 +111,8 @@ void launch_pool_update(const void* kc, const void* vc, void* kp, void* vp, cons
 // accumulating its columns for all heads of the workgroup, so a value row is read once per workgroup.
 template <typename T, int NWT, int NR2>
 __global__ void pool_window_attn_kernel(const float* __restrict__ q, const T* __restrict__ kc,
-                                        const T* __restrict__ vc, const float* __restrict__ kp,
-                                        const float* __restrict__ vp, const int* __restrict__ bt, int maxb,
+                                        const T* __restrict__ vc, const T* __restrict__ kp,
+                                        const T* __restrict__ vp, const int* __restrict__ bt, int maxb,
                                         const int* __restrict__ cu, const int* __restrict__ ctx,
                                         const float* __restrict__ pb, void* __restrict__ out, int out_f32, int B, int H,
                                         int G, int dim, int vdim, int bs, float scale, int window, int pool, int per,
@@ -167,8 +168,8 @@ __global__ void pool_window_attn_kernel(const float* __restrict__ q, const T* __
       for (int e = threadIdx.x; e < nk * dim; e += blockDim.x) {
         const int kk = e / dim, d = e - kk * dim;
         const int64_t sr = srow[kk];
-        tile[(size_t)kk * Dp + d] = sr < 0 ? kp[(-1 - sr) * krow + (int64_t)g * dim + d]
-                                           : El<T>::ld(kc + sr * krow + (int64_t)g * dim + d);
+        tile[(size_t)kk * Dp + d] = El<T>::ld(sr < 0 ? kp + (-1 - sr) * krow + (int64_t)g * dim + d
+                                                     : kc + sr * krow + (int64_t)g * dim + d);
       }
       __syncthreads();
       if (live) {
@@ -199,7 +200,7 @@ __global__ void pool_window_attn_kernel(const float* __restrict__ q, const T* __
             float v = 0.f;
             if (c < RV) {
               const int64_t col = (int64_t)g * vdim + v0 + c;
-              v = sr < 0 ? vp[(-1 - sr) * vrow + col] : El<T>::ld(vc + sr * vrow + col);
+              v = El<T>::ld(sr < 0 ? vp + (-1 - sr) * vrow + col : vc + sr * vrow + col);
             }
             vv[j][i] = v;
           }
@@ -255,7 +256,7 @@ static void pool_window_attn_t(const void* q, const void* kc, const void* vc, co
   dim3 g(T_, G * hchunks, zch);
 #define LAUNCH_PW(NW_, NR_)                                                                                         \
   pool_window_attn_kernel<T, NW_, NR_><<<g, NW_ * 64, bytes(KB), st>>>(                                             \
-      (const float*)q, (const T*)kc, (const T*)vc, (const float*)kp, (const float*)vp, (const int*)bt, maxb,        \
+      (const float*)q, (const T*)kc, (const T*)vc, (const T*)kp, (const T*)vp, (const int*)bt, maxb,                \
       (const int*)cu, (const int*)ctx, (const float*)pb, out, out_f32, B, H, G, dim, vdim, bs, scale, window, pool, \
       per, KB, Dp, hchunks, RVchunk)
 #define LAUNCH_PW_NR(NW_)                \
@@ -287,4 +288,292 @@ void launch_pool_window_attn(const void* q, const void* kc, const void* vc, cons
   DISPATCH_T(dt, T, (pool_window_attn_t<T>(q, kc, vc, kp, vp, bt, maxb, cu, ctx, pb, out, out_f32, T_, B, H, G, dim,
                                            vdim, bs, scale, window, pool, per, st)));
   HIP_CHECK_LAUNCH();
+}
+
+// The same attention on the matrix cores, for bf16 pages with key size 32, 64 or 128 and a value size that is a
+// multiple of 8: prompt portions and single rows alike. One workgroup serves one key/value group, GE of its query
+// heads and 64 * NS / GE query rows of one sequence: its 64 * NS slots enumerate (row, head) pairs, slot s -> row
+// s / GE, head s % GE, so a key tile is staged in LDS once for the whole head group. The rows' visible keys are
+// numbered u = 0 .. nb + ntok - 1 for the workgroup: first the pooled blocks the LAST row sees, then the positions
+// from the FIRST row's window start to the last row; a tile is 64 of them, whatever they are, and the mask tells each
+// row which of them it sees. Products are the swapped ones,
+//   S^T[key][slot] = K . Q^T   (A = K rows from LDS, B = Q^T fragments in registers)
+//   O^T[c][slot]  += V^T . P^T (A = V^T by transposing LDS reads, B = P^T straight from the S^T accumulators)
+// with the fp32 queries and the fp32 weights entering as value + remainder (two bf16 numbers, two matrix
+// instructions), so scores and weighted sums are those of 32-bit operands. There is no softmax: a weight is
+// sigmoid(score + bias) and the sums over keys are plain sums - so the keys can be split over workgroups at will
+// (nsplit > 1: each writes its partial sums, fp32, and pool_attn_reduce adds them in order), which is what gives a
+// step of single rows enough workgroups. The next tile's 16-byte chunks are fetched into registers while this one is
+// computed from LDS.
+template <int DK, int NVT, int NS>
+__global__ __launch_bounds__(256, 2) void pool_window_attn_mfma_kernel(
+    const float* __restrict__ q, const bf16_t* __restrict__ kc, const bf16_t* __restrict__ vc,
+    const bf16_t* __restrict__ kp, const bf16_t* __restrict__ vp, const int* __restrict__ block_tables, int max_blocks,
+    const int* __restrict__ cu_q, const int* __restrict__ ctx_lens, const float* __restrict__ pb,
+    void* __restrict__ out, int out_f32, float* __restrict__ part, int nsplit, int64_t part_stride, int H, int G,
+    int GE, int vdim, int bs, float scale, int window, int pool, int per, int nvch) {
+  constexpr int BKV = 64;
+  constexpr int LDK = DK + 16;
+  constexpr int VCH = NVT * 16;
+  constexpr int LDV = VCH + 16;
+  __shared__ __attribute__((aligned(16))) bf16_t Ks[BKV * LDK];
+  __shared__ __attribute__((aligned(16))) bf16_t Vs[BKV * LDV];
+  const int rep = H / G;
+  const int rows_per_wg = 64 * NS / GE;
+  const int rb = blockIdx.x / nsplit, sp = blockIdx.x % nsplit, by = blockIdx.y, b = blockIdx.z;
+  const int vch = by % nvch, hy = by / nvch;
+  const int kvh = hy / (rep / GE);
+  const int h0 = kvh * rep + (hy % (rep / GE)) * GE;
+  const int t0 = cu_q[b], qlen = cu_q[b + 1] - t0;
+  const int r0 = rb * rows_per_wg;
+  if (r0 >= qlen || ctx_lens[b] <= 0) return;
+  const int p0 = ctx_lens[b] - qlen;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int li = lane & 15, g = lane >> 4;
+  const int v0 = vch * VCH;
+  const int64_t vrow = (int64_t)G * vdim;
+  const int voff = kvh * vdim + v0;
+  constexpr float kLog2e = 1.4426950408889634f;
+
+  int row[NS], hd[NS], qpos[NS];
+  bool valid[NS], grp_rows[NS];
+  float bias2[NS];
+  s16x8 qf[NS][DK / 32], ql[NS][DK / 32];
+  f32x4 o[NS][NVT];
+  bool wave_rows = false;
+#pragma unroll
+  for (int n = 0; n < NS; ++n) {
+    const int gs = (w * NS + n) * 16, slot = gs + li;
+    row[n] = r0 + slot / GE;
+    hd[n] = h0 + slot % GE;
+    valid[n] = slot < rows_per_wg * GE && row[n] < qlen;
+    qpos[n] = p0 + (valid[n] ? row[n] : 0);
+    grp_rows[n] = r0 + gs / GE < qlen && gs < rows_per_wg * GE;
+    wave_rows = wave_rows || grp_rows[n];
+    bias2[n] = pb[valid[n] ? hd[n] : h0] * kLog2e;
+    const float* qp = q + ((int64_t)(t0 + (valid[n] ? row[n] : 0)) * H + (valid[n] ? hd[n] : h0)) * DK + 8 * g;
+#pragma unroll
+    for (int ks = 0; ks < DK / 32; ++ks)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float x = qp[32 * ks + j];
+        const bf16_t hi = f2bf(x);
+        qf[n][ks][j] = (short)hi;
+        ql[n][ks][j] = (short)f2bf(x - bf2f(hi));
+      }
+#pragma unroll
+    for (int i = 0; i < NVT; ++i) o[n][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float scale2 = scale * kLog2e;
+  const int pf = p0 + r0, pl = p0 + min(qlen, r0 + rows_per_wg) - 1;  // positions of the first and last row
+  const int jlo = window > 0 ? max(0, pf - window + 1) : 0;
+  const int nb = (pool > 0 && window > 0 && pl - window + 1 >= pool) ? (pl - window + 1) / pool : 0;
+  const int total = nb + (pl - jlo + 1);
+  const int tiles = (total + BKV - 1) / BKV, tps = (tiles + nsplit - 1) / nsplit;
+  const int u_begin = sp * tps * BKV, u_end = min(total, (sp + 1) * tps * BKV);
+  const int* bt = block_tables + (int64_t)b * max_blocks;
+  constexpr int CHK = DK / 8, CHV = VCH / 8;
+  static_assert((BKV * CHK) % 256 == 0 && (BKV * CHV) % 256 == 0, "whole 16-byte chunks per thread");
+  constexpr int NCK = BKV * CHK / 256, NCV = BKV * CHV / 256;
+  u16x8 kr[NCK], vr[NCV];
+  // the cache row of visible key u: a pooled row (negative) or a page row
+  auto src_row = [&](int u) -> int64_t {
+    if (u < nb) return -1 - pool_row(bt, u, pool, bs, per);
+    const int j = jlo + (u - nb);
+    return (int64_t)bt[j / bs] * bs + j % bs;
+  };
+  auto load_tile = [&](int u0) {
+#pragma unroll
+    for (int j = 0; j < NCK; ++j) {
+      const int c = threadIdx.x + 256 * j;
+      const int64_t sl = src_row(min(u0 + c / CHK, total - 1));
+      const bf16_t* base = sl < 0 ? kp + ((-1 - sl) * G + kvh) * DK : kc + (sl * G + kvh) * DK;
+      kr[j] = *reinterpret_cast<const u16x8*>(base + (c % CHK) * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < NCV; ++j) {
+      const int c = threadIdx.x + 256 * j;
+      const int ch = c % CHV;
+      const int64_t sl = src_row(min(u0 + c / CHV, total - 1));
+      const bf16_t* base = sl < 0 ? vp + (-1 - sl) * vrow + voff : vc + sl * vrow + voff;
+      u16x8 val = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (v0 + ch * 8 < vdim) val = *reinterpret_cast<const u16x8*>(base + ch * 8);
+      vr[j] = val;
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int j = 0; j < NCK; ++j) {
+      const int c = threadIdx.x + 256 * j;
+      *reinterpret_cast<u16x8*>(&Ks[(c / CHK) * LDK + (c % CHK) * 8]) = kr[j];
+    }
+#pragma unroll
+    for (int j = 0; j < NCV; ++j) {
+      const int c = threadIdx.x + 256 * j;
+      *reinterpret_cast<u16x8*>(&Vs[(c / CHV) * LDV + (c % CHV) * 8]) = vr[j];
+    }
+  };
+  auto compute_tile = [&](int u0) {
+    f32x4 s[NS][4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+#pragma unroll
+      for (int n = 0; n < NS; ++n) s[n][kt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < DK / 32; ++ks) {
+        const s16x8 kf = *reinterpret_cast<const s16x8*>(&Ks[(kt * 16 + li) * LDK + 32 * ks + 8 * g]);
+#pragma unroll
+        for (int n = 0; n < NS; ++n) {
+          s[n][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[n][ks], s[n][kt], 0, 0, 0);
+          s[n][kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, ql[n][ks], s[n][kt], 0, 0, 0);
+        }
+      }
+    }
+    // S^T accumulators: lane (li, g) holds slot li's scores for the keys u0 + 16 kt + 4 g + i
+    s16x8 pf_[NS][2], pl_[NS][2];
+#pragma unroll
+    for (int n = 0; n < NS; ++n) {
+#pragma unroll
+      for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int u = u0 + kt * 16 + 4 * g + i;
+          bool vis = grp_rows[n] && u < u_end;
+          if (u < nb) {
+            vis = vis && u * pool + pool - 1 <= qpos[n] - window;
+          } else {
+            const int j = jlo + (u - nb);
+            vis = vis && j <= qpos[n] && (window == 0 || qpos[n] - j < window);
+          }
+          const float e = __builtin_amdgcn_exp2f(-fmaf(s[n][kt][i], scale2, bias2[n]));
+          const float p = vis ? __builtin_amdgcn_rcpf(1.0f + e) : 0.f;
+          const bf16_t hi = f2bf(p);
+          pf_[n][kt >> 1][(kt & 1) * 4 + i] = (short)hi;
+          pl_[n][kt >> 1][(kt & 1) * 4 + i] = (short)f2bf(p - bf2f(hi));
+        }
+    }
+    const int tq = li >> 2, tp = li & 3;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+      for (int dt = 0; dt < NVT; ++dt) {
+        const bf16_t* a0 = &Vs[(32 * ks + 4 * g + tq) * LDV + dt * 16 + 4 * tp];
+        const bf16_t* a1 = a0 + 16 * LDV;
+        const s16x4 x0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(a0));
+        const s16x4 x1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_AS s16x4*)(a1));
+        const s16x8 vf = {x0[0], x0[1], x0[2], x0[3], x1[0], x1[1], x1[2], x1[3]};
+#pragma unroll
+        for (int n = 0; n < NS; ++n) {
+          o[n][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf_[n][ks], o[n][dt], 0, 0, 0);
+          o[n][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pl_[n][ks], o[n][dt], 0, 0, 0);
+        }
+      }
+    }
+  };
+  if (u_end > u_begin) load_tile(u_begin);
+  for (int u0 = u_begin; u0 < u_end; u0 += BKV) {
+    __syncthreads();  // every wave is done reading the previous tile
+    store_tile();
+    __syncthreads();
+    if (u0 + BKV < u_end) load_tile(u0 + BKV);
+    if (wave_rows) compute_tile(u0);
+  }
+#pragma unroll
+  for (int n = 0; n < NS; ++n) {
+    if (!valid[n]) continue;
+    const int64_t at = ((int64_t)(t0 + row[n]) * H + hd[n]) * vdim + v0 + 4 * g;
+#pragma unroll
+    for (int dt = 0; dt < NVT; ++dt) {
+      if (v0 + dt * 16 + 4 * g >= vdim) continue;
+      const f32x4 v = o[n][dt];
+      if (nsplit > 1) {
+        *reinterpret_cast<f32x4*>(part + (int64_t)sp * part_stride + at + dt * 16) = v;
+      } else if (out_f32) {
+        *reinterpret_cast<f32x4*>((float*)out + at + dt * 16) = v;
+      } else {
+        *reinterpret_cast<u16x4*>((bf16_t*)out + at + dt * 16) = u16x4{f2bf(v[0]), f2bf(v[1]), f2bf(v[2]), f2bf(v[3])};
+      }
+    }
+  }
+}
+
+// out[e] = sum over the splits, in order, of part[sp, e]; n a multiple of 4
+__global__ __launch_bounds__(256) void pool_attn_reduce_kernel(const float* __restrict__ part, int nsplit,
+                                                               int64_t stride, void* __restrict__ out, int out_f32,
+                                                               int64_t n) {
+  const int64_t e = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (e >= n) return;
+  f32x4 a = *reinterpret_cast<const f32x4*>(part + e);
+  for (int sp = 1; sp < nsplit; ++sp) a += *reinterpret_cast<const f32x4*>(part + (int64_t)sp * stride + e);
+  if (out_f32) *reinterpret_cast<f32x4*>((float*)out + e) = a;
+  else *reinterpret_cast<u16x4*>((bf16_t*)out + e) = u16x4{f2bf(a[0]), f2bf(a[1]), f2bf(a[2]), f2bf(a[3])};
+}
+
+bool pool_attn_mfma_ok(int dim, int vdim) { return (dim == 32 || dim == 64 || dim == 128) && vdim % 8 == 0; }
+
+// B sequences whose portions have at most max_qlen rows; rows [row0, row0 + rows) of `out` are theirs. nsplit > 1:
+// `part` holds nsplit * rows * H * vdim floats.
+void launch_pool_window_attn_mfma(const void* q, const void* kc, const void* vc, const void* kp, const void* vp,
+                                  const void* bt, int maxb, const void* cu, const void* ctx, const void* pb, void* out,
+                                  int out_f32, void* part, int nsplit, int64_t row0, int64_t rows, int B, int max_qlen,
+                                  int H, int G, int dim, int vdim, int bs, float scale, int window, int pool, int per,
+                                  hipStream_t st) {
+  if (B == 0 || max_qlen <= 0 || rows <= 0) return;
+  if (G < 1 || H % G) throw std::runtime_error("pool_window_attn: heads must be a multiple of the key/value heads");
+  if (!pool_attn_mfma_ok(dim, vdim)) throw std::runtime_error("pool_window_attn: shape not built for the matrix cores");
+  if (window < 0 || pool < 0 || (pool > 0 && (window == 0 || per < (bs + pool - 1) / pool)) || nsplit < 1)
+    throw std::runtime_error("pool_window_attn: bad window / pool / split");
+  const int rep = H / G;
+  int GE = 1;
+  for (int ge = std::min(rep, 64); ge >= 1; --ge)
+    if (rep % ge == 0) {
+      GE = ge;
+      break;
+    }
+  const int nvt = vdim > 128 ? 16 : (vdim > 64 ? 8 : 4);
+  const int nvch = (vdim + nvt * 16 - 1) / (nvt * 16);
+  const bool two_fit = nvt <= 4 || (nvt == 8 && dim != 128);
+  const int ns = (two_fit && max_qlen > 64 / GE) ? 2 : 1;
+  const int rows_per_wg = 64 * ns / GE;
+  const int64_t gy = (int64_t)G * (rep / GE) * nvch;
+  const int64_t gx = (int64_t)((max_qlen + rows_per_wg - 1) / rows_per_wg) * nsplit;
+  if (gy > 65535 || B > 65535 || gx > 0x7fffffff) throw std::runtime_error("pool_window_attn: grid too large");
+  dim3 grid((unsigned)gx, (unsigned)gy, B);
+  const int64_t stride = rows * H * vdim;
+  // partial sums are addressed by the step's row numbers: shift the base so that row0 lands on the buffer's start
+  float* pbase = part ? (float*)part - row0 * H * vdim : nullptr;
+#define LAUNCH_PWM(DK_, NVT_, NS_)                                                                                  \
+  pool_window_attn_mfma_kernel<DK_, NVT_, NS_><<<grid, 256, 0, st>>>(                                               \
+      (const float*)q, (const bf16_t*)kc, (const bf16_t*)vc, (const bf16_t*)kp, (const bf16_t*)vp, (const int*)bt,  \
+      maxb, (const int*)cu, (const int*)ctx, (const float*)pb, out, out_f32, pbase, nsplit, stride, H, G, GE, vdim, \
+      bs, scale, window, pool, per, nvch)
+#define LAUNCH_PWM_D(DK_)                     \
+  do {                                        \
+    if (nvt == 16) LAUNCH_PWM(DK_, 16, 1);    \
+    else if (nvt == 8) {                      \
+      if (ns == 2) LAUNCH_PWM(DK_, 8, 2);     \
+      else LAUNCH_PWM(DK_, 8, 1);             \
+    } else {                                  \
+      if (ns == 2) LAUNCH_PWM(DK_, 4, 2);     \
+      else LAUNCH_PWM(DK_, 4, 1);             \
+    }                                         \
+  } while (0)
+  if (dim == 32) LAUNCH_PWM_D(32);
+  else if (dim == 64) LAUNCH_PWM_D(64);
+  else {
+    if (nvt == 16) LAUNCH_PWM(128, 16, 1);
+    else if (nvt == 8) LAUNCH_PWM(128, 8, 1);
+    else if (ns == 2) LAUNCH_PWM(128, 4, 2);
+    else LAUNCH_PWM(128, 4, 1);
+  }
+#undef LAUNCH_PWM_D
+#undef LAUNCH_PWM
+  HIP_CHECK_LAUNCH();
+  if (nsplit > 1) {
+    const int64_t n = stride;
+    char* obase = (char*)out + row0 * H * vdim * (out_f32 ? 4 : 2);
+    pool_attn_reduce_kernel<<<(unsigned)((n / 4 + 255) / 256), 256, 0, st>>>((const float*)part, nsplit, stride, obase,
+                                                                            out_f32, n);
+    HIP_CHECK_LAUNCH();
+  }
 }

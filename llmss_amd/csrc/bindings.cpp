@@ -146,6 +146,12 @@ void launch_rope_pairs_cache(const void* proj, int64_t ldp, int off_q, int off_k
 void launch_pool_update(const void* kc, const void* vc, void* kp, void* vp, const void* bt, int maxb, const void* cu,
                         const void* ctx, int B, int max_qlen, int nk, int nv, int bs, int pool, int per, int dt,
                         hipStream_t st);
+bool pool_attn_mfma_ok(int dim, int vdim);
+void launch_pool_window_attn_mfma(const void* q, const void* kc, const void* vc, const void* kp, const void* vp,
+                                  const void* bt, int maxb, const void* cu, const void* ctx, const void* pb, void* out,
+                                  int out_f32, void* part, int nsplit, int64_t row0, int64_t rows, int B, int max_qlen,
+                                  int H, int G, int dim, int vdim, int bs, float scale, int window, int pool, int per,
+                                  hipStream_t st);
 void launch_pool_window_attn(const void* q, const void* kc, const void* vc, const void* kp, const void* vp,
                              const void* bt, int maxb, const void* cu, const void* ctx, const void* pb, void* out,
                              int out_f32, int T_, int B, int H, int G, int dim, int vdim, int bs, float scale,
@@ -506,6 +512,16 @@ PYBIND11_MODULE(_C, m) {
                                int per, int dt, uintptr_t st) {
     launch_pool_window_attn(CP(q), CP(kc), CP(vc), CP(kp), CP(vp), CP(bt), maxb, CP(cu), CP(ctx), CP(pb), P(out),
                             out_f32, T, B, H, G, dim, vdim, bs, scale, window, pool, per, dt, S(st));
+  });
+  m.def("pool_attn_mfma_ok", &pool_attn_mfma_ok);
+  m.def("pool_window_attn_mfma", [](uintptr_t q, uintptr_t kc, uintptr_t vc, uintptr_t kp, uintptr_t vp, uintptr_t bt,
+                                    int maxb, uintptr_t cu, uintptr_t ctx, uintptr_t pb, uintptr_t out, int out_f32,
+                                    uintptr_t part, int nsplit, int64_t row0, int64_t rows, int B, int max_qlen, int H,
+                                    int G, int dim, int vdim, int bs, float scale, int window, int pool, int per,
+                                    uintptr_t st) {
+    launch_pool_window_attn_mfma(CP(q), CP(kc), CP(vc), CP(kp), CP(vp), CP(bt), maxb, CP(cu), CP(ctx), CP(pb), P(out),
+                                 out_f32, P(part), nsplit, row0, rows, B, max_qlen, H, G, dim, vdim, bs, scale, window,
+                                 pool, per, S(st));
   });
   register_runtime(m);
   register_comm(m);

@@ -277,15 +277,15 @@ class PoolAttention:
         dt, dev = model.dtype, model.device
         per = PoolAttention.pooled_per_page(spec, block_size)
         pooled = {}
-        if per:  # fp32 means, row (page of the block's first position, rank of the block among those starting there)
-            pooled = {"kp": torch.zeros(num_blocks, per, spec.kv_heads * spec.dim, dtype=torch.float32, device=dev),
-                      "vp": torch.zeros(num_blocks, per, spec.kv_heads * spec.vdim, dtype=torch.float32, device=dev)}
+        if per:  # the blocks' means: row (page of the block's first position, rank among the blocks starting there)
+            pooled = {"kp": torch.zeros(num_blocks, per, spec.kv_heads * spec.dim, dtype=dt, device=dev),
+                      "vp": torch.zeros(num_blocks, per, spec.kv_heads * spec.vdim, dtype=dt, device=dev)}
         return (torch.zeros(num_blocks, block_size, spec.kv_heads * spec.dim, dtype=dt, device=dev),
                 torch.zeros(num_blocks, block_size, spec.kv_heads * spec.vdim, dtype=dt, device=dev), pooled)
 
     @staticmethod
-    def extra_bytes_per_block(spec, block_size: int) -> int:
-        return 4 * PoolAttention.pooled_per_page(spec, block_size) * spec.kv_heads * (spec.dim + spec.vdim)
+    def extra_bytes_per_block(spec, block_size: int, elem: int) -> int:
+        return elem * PoolAttention.pooled_per_page(spec, block_size) * spec.kv_heads * (spec.dim + spec.vdim)
 
     @staticmethod
     def forward(model: "LayeredLM", i: int, W, spec, h, inp: StepInput, cu, caches):
@@ -303,7 +303,7 @@ class PoolAttention:
         y = ops.pool_window_attn(q, kc, vc, kp, vp, inp.block_tables, cu, inp.ctx_lens, W.pb, spec.heads,
                                  spec.kv_heads, spec.dim, spec.vdim, spec.scale, spec.window, spec.pool, dt,
                                  max_qlen=1 if single else max(1, inp.max_seqlen),
-                                 num_decode=0 if single else inp.num_decode)
+                                 num_decode=0 if single else inp.num_decode, max_ctx=inp.max_ctx)
         return ops.linear_f(y, W.o, dt)
 
 
@@ -424,7 +424,8 @@ class LayeredLM:
 
     def kv_bytes_per_block(self, block_size: int) -> int:
         n = sum(block_size * r * self.w.wte.element_size() for r in self._cache_rows() if r)
-        n += sum(MIXERS[s.mixer.kind].extra_bytes_per_block(s.mixer, block_size) for s in self._run_specs()
+        n += sum(MIXERS[s.mixer.kind].extra_bytes_per_block(s.mixer, block_size, self.w.wte.element_size())
+                 for s in self._run_specs()
                  if hasattr(MIXERS[s.mixer.kind], "extra_bytes_per_block"))
         return max(1, n)
 

@@ -1569,8 +1569,9 @@ def _pool_caches(k_cache, v_cache, kp_cache, vp_cache, pool):
     bs = k_cache.shape[1]
     per = -(-bs // pool)
     for c, full, nm in ((kp_cache, k_cache, "pooled keys"), (vp_cache, v_cache, "pooled values")):
-        _f32c(c, nm)
-        _check(tuple(c.shape) == (full.shape[0], per, full.shape[2]), f"{nm} fp32 [blocks, ceil(block_size / pool), n]")
+        _check(c.is_cuda and c.is_contiguous() and c.dtype == full.dtype
+               and tuple(c.shape) == (full.shape[0], per, full.shape[2]),
+               f"{nm} [blocks, ceil(block_size / pool), n] in the pages' storage type")
     return per
 
 
@@ -1588,8 +1589,23 @@ def pool_update(k_cache, v_cache, kp_cache, vp_cache, block_tables, cu, ctx_lens
                       _dt(k_cache, "k cache"), _stream())
 
 
+_POOL_MFMA = os.environ.get("LLMSS_POOL_MFMA", "1") != "0"  # 0: every shape on the vector kernel (A/B runs)
+
+
+def pool_key_split(B: int, kv_heads: int, window: int, pool: int, max_ctx: int) -> int:
+    """Workgroups that share a single row's visible keys (at most min(window, max_ctx) positions and max_ctx / pool
+    pooled blocks): about 1024 workgroups in flight, whole 64-key tiles per split, at most 16 splits."""
+    keys = min(window, max_ctx) + (max_ctx // pool if pool else 0) if window > 0 else max_ctx
+    tiles = -(-max(keys, 1) // 64)
+    return max(1, min(tiles, 16, 1024 // max(1, B * kv_heads)))
+
+
 def pool_window_attn(q, k_cache, v_cache, kp_cache, vp_cache, block_tables, cu, ctx_lens, pb, heads, kv_heads, dim,
-                     vdim, scale, window, pool, out_dtype, max_qlen=0, num_decode=0):
+                     vdim, scale, window, pool, out_dtype, max_qlen=0, num_decode=0, max_ctx=0):
+    """``max_qlen`` (the longest portion of the step, known on the host) > 0: bf16 pages of a shape the matrix-core
+    kernel is built for run on it, the ``num_decode`` leading single-row sequences in one launch - their keys split
+    over workgroups when ``max_ctx`` (an upper bound of every context length) is given - and the portions in
+    another; everything else runs the vector kernel."""
     T = q.shape[0]
     _rows(q, "q", heads * dim, torch.float32)
     _check(q.is_contiguous(), "q contiguous")
@@ -1603,6 +1619,27 @@ def pool_window_attn(q, k_cache, v_cache, kp_cache, vp_cache, block_tables, cu, 
     _f32c(pb, "pb")
     _check(pb.numel() == heads and out_dtype in _DT, "pb [heads]; out bf16 / fp32")
     out = torch.empty(T, heads * vdim, dtype=out_dtype, device=q.device)
+    nd = int(num_decode)
+    _check(0 <= nd <= B, "num_decode outside the step")
+    al = lambda t: t is None or t.data_ptr() % 16 == 0
+    if (k_cache.dtype == torch.bfloat16 and max_qlen > 0 and _POOL_MFMA and lib().pool_attn_mfma_ok(dim, vdim)
+            and al(k_cache) and al(v_cache) and (not pool or (al(kp_cache) and al(vp_cache)))):
+        maxb = block_tables.shape[1]
+        for first, n, ql in ((0, nd, 1), (nd, B - nd, int(max_qlen))):
+            if n <= 0:
+                continue
+            row0 = 0 if first == 0 else nd  # single-row sequences come first: sequence b's row is row b
+            rows = n if ql == 1 else T - row0
+            nsplit = pool_key_split(n, kv_heads, int(window), int(pool), int(max_ctx)) if ql == 1 and max_ctx > 0 else 1
+            part = torch.empty(nsplit, rows, heads * vdim, dtype=torch.float32, device=q.device) if nsplit > 1 else None
+            lib().pool_window_attn_mfma(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                        _ptr(kp_cache) if pool else 0, _ptr(vp_cache) if pool else 0,
+                                        block_tables.data_ptr() + 4 * first * maxb, maxb, cu.data_ptr() + 4 * first,
+                                        ctx_lens.data_ptr() + 4 * first, pb.data_ptr(), out.data_ptr(),
+                                        int(out_dtype == torch.float32), _ptr(part), nsplit, row0, rows, n, ql, heads,
+                                        kv_heads, dim, vdim, k_cache.shape[1], float(scale), int(window), int(pool),
+                                        per, _stream())
+        return out
     lib().pool_window_attn(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _ptr(kp_cache) if pool else 0,
                            _ptr(vp_cache) if pool else 0, block_tables.data_ptr(), block_tables.shape[1], cu.data_ptr(),
                            ctx_lens.data_ptr(), pb.data_ptr(), out.data_ptr(), int(out_dtype == torch.float32), T, B,

@@ -1022,9 +1022,9 @@ def pool_slot(block_tables, b: int, blk: int, pool: int, bs: int, per: int):
 
 
 def pool_update(k_cache, v_cache, kp_cache, vp_cache, block_tables, cu, ctx_lens, pool: int, max_qlen: int = 0):
-    """Mean key and mean value (fp32) of every block of ``pool`` positions whose last position the step has just
-    written, from the cached rows of the block: kp_cache / vp_cache fp32 [blocks, ceil(block_size / pool), kv_heads *
-    dim | vdim], row :func:`pool_slot`. ``max_qlen`` (the step's longest portion) only sizes the GPU kernel's grid."""
+    """Mean key and mean value (formed in fp32) of every block of ``pool`` positions whose last position the step has
+    just written, from the cached rows of the block: kp_cache / vp_cache [blocks, ceil(block_size / pool), kv_heads *
+    dim | vdim] in the pages' storage type, row :func:`pool_slot`. ``max_qlen`` (the step's longest portion) only sizes the GPU kernel's grid."""
     bs, per = k_cache.shape[1], kp_cache.shape[1]
     nk, nv = k_cache.shape[2], v_cache.shape[2]
     for b, _, n, p0 in _seq_rows(cu, ctx_lens):
@@ -1033,17 +1033,17 @@ def pool_update(k_cache, v_cache, kp_cache, vp_cache, block_tables, cu, ctx_lens
             pos = torch.arange(blk * pool, blk * pool + pool)
             rows = block_tables[b, pos // bs].long() * bs + pos % bs
             s = pool_slot(block_tables, b, blk, pool, bs, per)
-            kp_cache.view(-1, nk)[s] = k_cache.view(-1, nk)[rows].float().mean(0)
-            vp_cache.view(-1, nv)[s] = v_cache.view(-1, nv)[rows].float().mean(0)
+            kp_cache.view(-1, nk)[s] = k_cache.view(-1, nk)[rows].float().mean(0).to(kp_cache.dtype)
+            vp_cache.view(-1, nv)[s] = v_cache.view(-1, nv)[rows].float().mean(0).to(vp_cache.dtype)
 
 
 def pool_window_attn(q, k_cache, v_cache, kp_cache, vp_cache, block_tables, cu, ctx_lens, pb, heads: int,
                      kv_heads: int, dim: int, vdim: int, scale: float, window: int, pool: int, out_dtype,
-                     max_qlen: int = 0, num_decode: int = 0):
+                     max_qlen: int = 0, num_decode: int = 0, max_ctx: int = 0):
     """Sigmoid-weighted attention of every row over its sequence's cache: the row at position i adds sigmoid(q . k *
     scale + pb[head]) * v over the positions j with 0 <= i - j (< window when window > 0) and, when ``pool`` > 0, over
     the pooled rows of the blocks with blk * pool + pool - 1 <= i - window. q fp32 [T, heads * dim]; returns [T, heads
-    * vdim] in ``out_dtype``. ``max_qlen`` and ``num_decode`` only steer the GPU kernels."""
+    * vdim] in ``out_dtype``. ``max_qlen``, ``num_decode`` and ``max_ctx`` only steer the GPU kernels."""
     T = q.shape[0]
     bs = k_cache.shape[1]
     rep = heads // kv_heads

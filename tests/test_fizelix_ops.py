@@ -130,7 +130,7 @@ def test_token_side_add(device, dtype, W, d, part):
 
 # -------------------------------------------------------------------------- windowed sigmoid attention, pooled blocks
 def run_attention(device, dtype, lens, cuts, H, G, dim, vdim, window, pool, rot, bs=16, seed=0, q=None, k=None, v=None,
-                  scale=0.3, pb=None):
+                  scale=0.3, pb=None, max_ctx=0):
     """Feeds q / k / v rows of several sequences through rope_pairs_cache, pool_update and pool_window_attn step by
     step (portions as ``cuts`` says, all sequences of a step in one batch) and returns per sequence (got, want)."""
     S = len(lens)
@@ -144,8 +144,8 @@ def run_attention(device, dtype, lens, cuts, H, G, dim, vdim, window, pool, rot,
     kc = torch.full((pages.blocks, bs, G * dim), 7.0, dtype=dtype, device=device)  # stale values everywhere
     vc = torch.full((pages.blocks, bs, G * vdim), -3.0, dtype=dtype, device=device)
     per = -(-bs // pool) if pool else 0
-    kp = torch.full((pages.blocks, per, G * dim), 5.0, device=device) if pool else None
-    vp = torch.full((pages.blocks, per, G * vdim), 5.0, device=device) if pool else None
+    kp = torch.full((pages.blocks, per, G * dim), 5.0, dtype=dtype, device=device) if pool else None
+    vp = torch.full((pages.blocks, per, G * vdim), 5.0, dtype=dtype, device=device) if pool else None
     freqs = torch.tensor([base ** (-2.0 * i / rot) for i in range(rot // 2)], dtype=torch.float32, device=device) if rot else None
     got = [torch.zeros(n, H * vdim, dtype=F64) for n in lens]
     for step in steps_of(cuts):
@@ -161,7 +161,7 @@ def run_attention(device, dtype, lens, cuts, H, G, dim, vdim, window, pool, rot,
         if pool:
             ops.pool_update(kc, vc, kp, vp, bt, cu, ctx, pool, max_qlen=mq)
         out = ops.pool_window_attn(qq, kc, vc, kp, vp, bt, cu, ctx, pb.float().to(device), H, G, dim, vdim, scale,
-                                   window, pool, torch.float32, max_qlen=mq)
+                                   window, pool, torch.float32, max_qlen=mq, max_ctx=max_ctx)
         at = 0
         for s, p0, n in step:
             got[s][p0:p0 + n] = out[at:at + n].double().cpu()
@@ -186,33 +186,42 @@ def run_attention(device, dtype, lens, cuts, H, G, dim, vdim, window, pool, rot,
     (2, 2, 10, 6, 40, 8, 0),     # a window longer than most of the prompt
     (2, 1, 8, 8, 0, 0, 4),       # no window, no pool: every earlier position
     (2, 2, 8, 8, 6, 0, 0),       # a window without pooled blocks
+    (4, 2, 32, 64, 7, 3, 8),     # sizes the matrix-core kernel takes (bf16 pages): two slot groups per wave
+    (8, 2, 64, 24, 12, 5, 64),   # four heads to a key head, a value size that is no multiple of 16
+    (4, 1, 128, 128, 9, 16, 32),  # the widest key, one slot group
+    (2, 2, 64, 136, 20, 1, 0),   # a value row in the widest tile, blocks of one position
+    (3, 1, 32, 8, 0, 0, 16),     # three heads to a key head, every earlier position
 ])
 def test_attention_portions_batches(device, dtype, H, G, dim, vdim, window, pool, rot):
     lens = [45, 23, 1, 38]
     cuts = [[45], [2, 2, 3, 16], [1], [30, 1, 1, 1, 1, 1, 1, 1, 1]]  # whole, small portions, one token, prompt + decoding
-    for got, want in run_attention(device, dtype, lens, cuts, H, G, dim, vdim, window, pool, rot):
-        close(got, want, dtype, "attention rows", slack=1.0 if dtype == torch.float32 else 2.0)
+    for max_ctx in (0, 4096):  # with a bound on the context a step of single rows splits their keys over workgroups
+        for got, want in run_attention(device, dtype, lens, cuts, H, G, dim, vdim, window, pool, rot, max_ctx=max_ctx,
+                                       scale=0.3 * (8.0 / dim) ** 0.5):
+            close(got, want, dtype, "attention rows", slack=1.0 if dtype == torch.float32 else 2.0)
 
 
 @pytest.mark.parametrize("device,dtype", RUNS)
 @pytest.mark.parametrize("decode", [False, True])
-def test_attention_standout_key(device, dtype, decode):
+@pytest.mark.parametrize("dim,vdim", [(8, 4), (32, 8)])
+def test_attention_standout_key(device, dtype, decode, dim, vdim):
     """One key is made to match the last row's query far better than any other; its value is unlike every other. Where
     it sits decides what the last row must return: inside the window its own value, in a pooled block a P-th of it
     (through the block's mean key), in a block not yet pooled and already outside the window nothing at all."""
-    H, G, dim, vdim, window, pool, n = 2, 1, 8, 4, 10, 4, 90
+    H, G, window, pool, n = 2, 1, 10, 4, 90
     for place in (0, 3, 4, 15, 16, 17, 63, 64, 71, 72, 75, 76, 79, 80, 81, 89):
         q, k, v = rnd(n, H * dim, seed=1, mul=0.1), rnd(n, G * dim, seed=2, mul=0.1), rnd(n, G * vdim, seed=3, mul=0.1)
         k[place] = 0.0
-        k[place, :dim] = 4.0
+        k[place, :8] = 4.0
         q[n - 1] = 0.0
-        q[n - 1, :dim] = 4.0
-        q[n - 1, dim:] = 4.0
-        v[place] = torch.tensor([100.0, -50.0, 25.0, 10.0])
+        q[n - 1, :8] = 4.0
+        q[n - 1, dim:dim + 8] = 4.0
+        v[place] = 0.0
+        v[place, :4] = torch.tensor([100.0, -50.0, 25.0, 10.0], dtype=F64)
         cuts = [[n - 6] + [1] * 6] if decode else [[n - 30, 17, 11, 2]]
         (got, want), = run_attention(device, dtype, [n], cuts, H, G, dim, vdim, window, pool, 0, q=[q.to(dtype).double()],
                                      k=[k.to(dtype).double()], v=[v.to(dtype).double()], scale=0.5,
-                                     pb=torch.tensor([-6.0, -6.0], dtype=F64))
+                                     pb=torch.tensor([-6.0, -6.0], dtype=F64), max_ctx=128 if decode else 0)
         last = want[n - 1].view(H, vdim)[0, 0]
         i = n - 1
         if i - place < window:
