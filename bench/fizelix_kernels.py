@@ -101,21 +101,21 @@ def main():
         proj = rn(T, Np)
         kc, vc = rn(B * nblk, bs, nk), rn(B * nblk, bs, nk)
         per = -(-bs // pool)
-        kp, vp = f32(B * nblk, per, nk), f32(B * nblk, per, nk)
+        kp, vp = rn(B * nblk, per, nk), rn(B * nblk, per, nk)
         freqs = torch.tensor([10000.0 ** (-2.0 * i / (D // 2)) for i in range(D // 4)], device=dev)
         cs = ops.rope_angles(pos, freqs)
         t = timed(lambda: ops.rope_pairs_cache(proj, 0, nq, nq + nk, cs, kc, vc, slots, H, G, D, D))
         add("rope_pairs_cache", phase, t, bytes_=T * ((nq + 2 * nk) * 2 + nq * 4 + 2 * nk * 2))
         qf = ops.rope_pairs_cache(proj, 0, nq, nq + nk, cs, kc, vc, slots, H, G, D, D)
         t = timed(lambda: ops.pool_update(kc, vc, kp, vp, bt, cu, cl, pool, max_qlen=q))
-        add("pool_update", phase, t, bytes_=B * (q // pool + 1) * 2 * nk * (pool * 2 + 4))
+        add("pool_update", phase, t, bytes_=B * (q // pool + 1) * 2 * nk * (pool * 2 + 2))
         pb = f32(H)
         f_att = lambda: ops.pool_window_attn(qf, kc, vc, kp, vp, bt, cu, cl, pb, H, G, D, D, D ** -0.5, win, pool, bf,
-                                             max_qlen=q)
+                                             max_qlen=q, max_ctx=ctx if phase == "decode" else 0)
         t = timed(f_att, iters=3, warm=1)
         seen_tok, seen_blk = min(ctx, win), max(0, (ctx - win) // pool)
         add("pool_window_attn", phase, t, flops=pairs * H * 4 * D,
-            bytes_=(T * nq * 4 + B * 2 * nk * (seen_tok * 2 + seen_blk * 4) + T * nq * 2) if phase == "decode" else 0)
+            bytes_=(T * nq * 4 + B * 2 * nk * (seen_tok + seen_blk) * 2 + T * nq * 2) if phase == "decode" else 0)
         kc2, vc2 = rn(B * nblk, G, bs, D), rn(B * nblk, G, bs, D)
         if phase == "prompt":
             qkv = rn(T, (H + 2 * G) * D)

@@ -335,8 +335,8 @@ __global__ __launch_bounds__(256, 2) void pool_window_attn_mfma_kernel(
   const int voff = kvh * vdim + v0;
   constexpr float kLog2e = 1.4426950408889634f;
 
-  int row[NS], hd[NS], qpos[NS];
-  bool valid[NS], grp_rows[NS];
+  int row[NS], hd[NS], qpos[NS], grp_first[NS], grp_last[NS];
+  bool valid[NS], grp_rows[NS], grp_full[NS];
   float bias2[NS];
   s16x8 qf[NS][DK / 32], ql[NS][DK / 32];
   f32x4 o[NS][NVT];
@@ -349,6 +349,9 @@ __global__ __launch_bounds__(256, 2) void pool_window_attn_mfma_kernel(
     valid[n] = slot < rows_per_wg * GE && row[n] < qlen;
     qpos[n] = p0 + (valid[n] ? row[n] : 0);
     grp_rows[n] = r0 + gs / GE < qlen && gs < rows_per_wg * GE;
+    grp_full[n] = r0 + (gs + 15) / GE < qlen && gs + 15 < rows_per_wg * GE;  // every slot of the group holds a row
+    grp_first[n] = p0 + min(qlen - 1, r0 + gs / GE);  // (the same in every lane)
+    grp_last[n] = p0 + min(qlen - 1, r0 + (gs + 15) / GE);
     wave_rows = wave_rows || grp_rows[n];
     bias2[n] = pb[valid[n] ? hd[n] : h0] * kLog2e;
     const float* qp = q + ((int64_t)(t0 + (valid[n] ? row[n] : 0)) * H + (valid[n] ? hd[n] : h0)) * DK + 8 * g;
@@ -414,6 +417,26 @@ __global__ __launch_bounds__(256, 2) void pool_window_attn_mfma_kernel(
     }
   };
   auto compute_tile = [&](int u0) {
+    // what the tile is to each slot group: 0 nothing of it is seen (weights zero), 1 some of it (masked), 2 all of it
+    // by every row of the group (no mask). A tile of pooled rows and positions both is masked.
+    int see[NS];
+    bool any = false;
+    const int ul = u0 + BKV - 1;
+#pragma unroll
+    for (int n = 0; n < NS; ++n) {
+      see[n] = grp_rows[n] ? 1 : 0;
+      if (ul < nb) {  // pooled rows only
+        if (u0 * pool + pool - 1 > grp_last[n] - window) see[n] = 0;
+        else if (grp_full[n] && ul < u_end && ul * pool + pool - 1 <= grp_first[n] - window) see[n] = see[n] ? 2 : 0;
+      } else if (u0 >= nb) {  // positions only
+        const int j0 = jlo + (u0 - nb), j1 = j0 + BKV - 1;
+        if (j0 > grp_last[n] || (window > 0 && grp_first[n] - j1 >= window)) see[n] = 0;
+        else if (grp_full[n] && ul < u_end && j1 <= grp_first[n] && (window == 0 || grp_last[n] - j0 < window))
+          see[n] = see[n] ? 2 : 0;
+      }
+      any = any || see[n] != 0;
+    }
+    if (!any) return;
     f32x4 s[NS][4];
 #pragma unroll
     for (int kt = 0; kt < 4; ++kt) {
@@ -431,26 +454,40 @@ __global__ __launch_bounds__(256, 2) void pool_window_attn_mfma_kernel(
     }
     // S^T accumulators: lane (li, g) holds slot li's scores for the keys u0 + 16 kt + 4 g + i
     s16x8 pf_[NS][2], pl_[NS][2];
-#pragma unroll
-    for (int n = 0; n < NS; ++n) {
+    auto weights = [&](int n, auto whole_c) {
+      constexpr bool WHOLE = decltype(whole_c)::value;
 #pragma unroll
       for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          const int u = u0 + kt * 16 + 4 * g + i;
-          bool vis = grp_rows[n] && u < u_end;
-          if (u < nb) {
-            vis = vis && u * pool + pool - 1 <= qpos[n] - window;
-          } else {
-            const int j = jlo + (u - nb);
-            vis = vis && j <= qpos[n] && (window == 0 || qpos[n] - j < window);
-          }
           const float e = __builtin_amdgcn_exp2f(-fmaf(s[n][kt][i], scale2, bias2[n]));
-          const float p = vis ? __builtin_amdgcn_rcpf(1.0f + e) : 0.f;
+          float p = __builtin_amdgcn_rcpf(1.0f + e);
+          if constexpr (!WHOLE) {
+            const int u = u0 + kt * 16 + 4 * g + i;
+            bool vis = u < u_end;
+            if (u < nb) {
+              vis = vis && u * pool + pool - 1 <= qpos[n] - window;
+            } else {
+              const int j = jlo + (u - nb);
+              vis = vis && j <= qpos[n] && (window == 0 || qpos[n] - j < window);
+            }
+            p = vis ? p : 0.f;
+          }
           const bf16_t hi = f2bf(p);
           pf_[n][kt >> 1][(kt & 1) * 4 + i] = (short)hi;
           pl_[n][kt >> 1][(kt & 1) * 4 + i] = (short)f2bf(p - bf2f(hi));
         }
+    };
+#pragma unroll
+    for (int n = 0; n < NS; ++n) {
+      if (see[n] == 0) {
+        const s16x8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+        pf_[n][0] = pf_[n][1] = pl_[n][0] = pl_[n][1] = z;
+      } else if (see[n] == 2) {
+        weights(n, std::true_type{});
+      } else {
+        weights(n, std::false_type{});
+      }
     }
     const int tq = li >> 2, tp = li & 3;
 #pragma unroll
