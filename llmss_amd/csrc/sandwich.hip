@@ -189,7 +189,7 @@ __device__ __forceinline__ float gelu_tanh_f(float z) {
 
 // buf: [W] the x row, then [W] the projected row, then [d] the gated numbers
 template <typename T, int V>
-__global__ __launch_bounds__(256) void token_side_add_kernel(SandwichArgs p, SideArgs s) {
+__global__ __launch_bounds__(512) void token_side_add_kernel(SandwichArgs p, SideArgs s) {
   extern __shared__ __attribute__((aligned(16))) float buf[];
   __shared__ float red[16];
   const int t = blockIdx.x, W = p.W, d = s.d;
@@ -222,10 +222,23 @@ __global__ __launch_bounds__(256) void token_side_add_kernel(SandwichArgs p, Sid
   }
   __syncthreads();
   float ss = 0.f;
+  const bool rows16 = sizeof(T) == 2 && d % 8 == 0 && ((uintptr_t)s.wp & 15) == 0;  // 16-byte reads of a bf16 row
   for (int c = threadIdx.x; c < W; c += blockDim.x) {
     const T* wr = (const T*)s.wp + (int64_t)c * d;
-    float a = 0.f;
-    for (int j = 0; j < d; ++j) a = fmaf(El<T>::ld(wr + j), gs[j], a);
+    float a = 0.f, a2 = 0.f;
+    if (rows16) {
+      for (int j = 0; j < d; j += 8) {
+        const u16x8 w8 = *reinterpret_cast<const u16x8*>(wr + j);
+#pragma unroll
+        for (int i = 0; i < 8; i += 2) {
+          a = fmaf(bf2f(w8[i]), gs[j + i], a);
+          a2 = fmaf(bf2f(w8[i + 1]), gs[j + i + 1], a2);
+        }
+      }
+      a += a2;
+    } else {
+      for (int j = 0; j < d; ++j) a = fmaf(El<T>::ld(wr + j), gs[j], a);
+    }
     ys[c] = a;
     ss = fmaf(a, a, ss);
   }
@@ -267,8 +280,8 @@ void launch_token_side_add(void* x, const void* ids, const void* table, int64_t 
   const bool vec = W % 4 == 0 && al16(x) && al16(wn) && al16(add) && al16(wnext) && ((uintptr_t)wg % (4 * es)) == 0 &&
                    (!h || (((uintptr_t)h % (4 * es)) == 0 && ldh % 4 == 0));
   DISPATCH_T(dt, T, {
-    if (vec) token_side_add_kernel<T, 4><<<T_, 256, lds, st>>>(p, s);
-    else token_side_add_kernel<T, 1><<<T_, 256, lds, st>>>(p, s);
+    if (vec) token_side_add_kernel<T, 4><<<T_, 512, lds, st>>>(p, s);
+    else token_side_add_kernel<T, 1><<<T_, 512, lds, st>>>(p, s);
   });
   HIP_CHECK_LAUNCH();
 }
