@@ -213,7 +213,7 @@ def test_portions_of_several_sizes(cases, cuts, name, device, dtype):
 
 
 @pytest.mark.parametrize("device,dtype", RUNS)
-@pytest.mark.parametrize("name", ["mixed", "plain", "odd"])
+@pytest.mark.parametrize("name", ["mixed", "plain", "odd", "wide"])
 def test_mixed_batch_of_unequal_requests_equals_each_alone(cases, name, device, dtype):
     c = cases(name, device, dtype)
     seqs = {0: toks(50, c.V, 5), 1: toks(23, c.V, 6), 2: toks(9, c.V, 7), 3: toks(37, c.V, 8)}

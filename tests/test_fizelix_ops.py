@@ -191,6 +191,8 @@ def run_attention(device, dtype, lens, cuts, H, G, dim, vdim, window, pool, rot,
     (4, 1, 128, 128, 9, 16, 32),  # the widest key, one slot group
     (2, 2, 64, 136, 20, 1, 0),   # a value row in the widest tile, blocks of one position
     (3, 1, 32, 8, 0, 0, 16),     # three heads to a key head, every earlier position
+    (2, 1, 8, 8, 5, 20, 0),      # a block longer than a page (vector kernel)
+    (2, 1, 64, 32, 5, 20, 0),    # the same on the matrix cores
 ])
 def test_attention_portions_batches(device, dtype, H, G, dim, vdim, window, pool, rot):
     lens = [45, 23, 1, 38]
